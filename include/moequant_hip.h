@@ -1,0 +1,118 @@
+/* moequant_hip.h -- C ABI of libmoequant_hip.so (AMD gfx950 / MI355X).
+ *
+ * Conventions (all entry points):
+ *   - every pointer is a DEVICE pointer owned by the caller, including workspaces; the library never
+ *     allocates, frees or synchronises;
+ *   - every kernel is launched on `stream` (a hipStream_t passed as void*; NULL = the default stream);
+ *   - return value: 0 = launched, <0 = MQ_ERR_* (nothing launched, or launching stopped at the failing
+ *     kernel); numerical trouble is reported through a device-side `info` word, LAPACK style;
+ *   - matrices are row-major, `ld*` are leading dimensions in ELEMENTS;
+ *   - no exceptions cross the boundary; calls are re-entrant per stream.
+ *
+ * Citations name the MoE-Quant code each entry point replaces (paths relative to that repository).
+ */
+#ifndef MOEQUANT_HIP_H
+#define MOEQUANT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MQ_OK 0
+#define MQ_ERR_ARG (-1)
+#define MQ_ERR_LAUNCH (-2)
+#define MQ_ERR_WORKSPACE (-3)
+
+/* element types for `w_dtype` / `round_dtype` */
+#define MQ_DT_F32 0 /* round_dtype: no rounding */
+#define MQ_DT_BF16 1
+#define MQ_DT_F16 2
+
+/* ---- (1) Hessian accumulation -------------------------------------------------------------------
+ * H <- beta*H + alpha * X^T X.   Replaces `self.H.addmm_(input.T, input, beta, alpha)` together with
+ * the `input.float()` up-cast in GPTQ.update, src/gptq.py:97-103.
+ *   H  : C x C fp32 (ldh).  Only the upper triangle of the old H is read.  The upper triangle is always
+ *        written; with mirror != 0 the lower triangle is written too (symmetric copy).
+ *   X  : n x C bf16 (ldx), C and ldx even, X 4-byte aligned.   n == 0 just scales H by beta.
+ *   workspace: mq_hessian_syrk_workspace_bytes(n, C) bytes (0 when the tile count alone fills the GPU).
+ */
+size_t mq_hessian_syrk_workspace_bytes(int n, int C);
+int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
+                         int mirror, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- (2) damped Cholesky / Cholesky-inverse -------------------------------------------------------
+ * In place: A (SPD, upper triangle read, C % 128 == 0) -> unit-diagonal upper-triangular
+ * U = chol(A^-1, upper) / diag, strictly lower part zeroed.  Replaces
+ * `linalg_utils.inv_sym` (src/linalg_utils.py:8-12) + `torch.linalg.cholesky(H, upper=True)` +
+ * `H_inv_cho.div_(H_inv_cho.diag()[:, None])` in GPTQ._get_hessian_inverse, src/gptq.py:236-242.
+ *   normalize : 1 = rows divided by the diagonal (what the GPTQ loop wants); 0 = plain R^-1 = chol(A^-1, upper),
+ *          from which inv_sym assembles A^-1 = R^-T R^-1.
+ *   info : one device int, must be 0 on entry; a non-positive/NaN pivot stores its 1-based index
+ *          (the torch path raises LinAlgError there and the caller falls back to identity,
+ *          src/gptq.py:239-240).  The output is unspecified when info != 0.
+ */
+int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream);
+
+/* ---- (3) quantization grid and column loop ---------------------------------------------------------
+ * Symmetric per-group scales.  Replaces find_quantization_meta (symmetric branch) as called from
+ * get_quantization_grid, src/quant_utils.py:75-96,213-220:
+ *   scale = round_to(round_dtype)((2/maxq) * max|w| + 1e-12) over each group of `group_size` columns.
+ *   W : R x C (w_dtype, ldw); dead_cols (nullable, C bytes): columns treated as zero (src/gptq.py:152).
+ *   scale_rg : R x G fp32 out;  scale_gr (nullable): the same values transposed, G x R.
+ */
+int mq_quant_grid_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size, int bits,
+                      const uint8_t* dead_cols, int round_dtype, float* scale_rg, float* scale_gr, void* stream);
+
+/* Wt[j, r] = fp32(W[r, perm[j]]), 0 for dead columns.  Replaces `self.W.clone().float()`,
+ * `self.W[:, pruned_ids] = 0` (src/gptq.py:149-152) and `self.W.transpose(-2, -1)[perm]` (src/gptq.py:192).
+ * perm nullable = identity. */
+int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int* perm, const uint8_t* dead_cols,
+                  float* Wt, long ldwt, void* stream);
+
+/* The blocked GPTQ loop.  Replaces gptq_loop / gptq_loop_graph with both Triton kernels and the per-block
+ * addmm_, src/gptq_loop.py:12-40,68-88,141-148.
+ *   Wt    : C x R fp32 (ldw), in/out: original (permuted) weights in, dequantized weights out.
+ *   U     : C x C fp32 (ldu), unit-diagonal upper factor from mq_factor_upper_inverse (only k > j read).
+ *   scale : scale of (column j, row r) is scale[srow*ld_scale + r] with srow = scale_row ? scale_row[j] : j,
+ *           so both the replicated C x R array of the reference and a compact G x R array work.
+ *   qzero : nullable, same indexing; NULL means the constant qzero_const.
+ *   round_dtype : rounding of the dequantized value ((q - z) * s), the `dtype` of tl_dequantize.
+ *   block : columns per lazy-batch block; values <= 0 or > 128 use 128 (only reassociates fp32 sums).
+ *   Qt    : C x R u8 out, integer codes.   E : 128 x R fp32 scratch (error block).
+ */
+int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale, long ld_scale,
+                 const int* scale_row, const float* qzero, float qzero_const, float maxq, int round_dtype, int block,
+                 uint8_t* Qt, float* E, void* stream);
+
+/* codes[r, c] = Qt[perm_inv[c], r].  Replaces `[perm_inv].transpose(-2, -1).contiguous().to(torch.uint8)`,
+ * src/gptq.py:199.  perm_inv nullable = identity. */
+int mq_untranspose_codes(const uint8_t* Qt, int R, int C, const int* perm_inv, uint8_t* codes, long ldc,
+                         void* stream);
+
+/* ---- (4) int4 -> int32 packing (compressed_tensors "pack-quantized" layout) -------------------------
+ * word[r, k] = sum_{i<8} ((codes[r, 8k+i] - zero[r, (8k+i)/g] + 8) & 15) << 4i, columns past C pack as 0.
+ * Replaces pack_weight's `qweight.to(int8) - zero...` + compressed_tensors.pack_to_int32(., 4),
+ * pack_quantized_model.py:66-67.   zero (R x G fp32) nullable = 8 everywhere (symmetric).
+ * out : R x ceil(C/8) int32 (ldo).
+ */
+int mq_pack_int4(const uint8_t* codes, long ldc, int R, int C, const float* zero, int group_size, int32_t* out,
+                 long ldo, void* stream);
+
+/* Same words, straight from the loop's transposed codes (symmetric, zero = 8): fuses mq_untranspose_codes
+ * and mq_pack_int4 so the codes are read once. */
+int mq_pack_from_qt(const uint8_t* Qt, int R, int C, const int* perm_inv, int32_t* out, long ldo, void* stream);
+
+/* ---- building block, exported for tests -----------------------------------------------------------
+ * C[m,n] = beta*C[m,n] + alpha * sum_k A(m,k) B(k,n) on the fp32 matrix cores; A(m,k) = A[m*sam + k*sak]
+ * (one of sam/sak must be 1), B(k,n) = B[k*sbk + n*sbn] likewise.  tri != 0: only 128x128 tiles on or above
+ * the block diagonal.  ktrim: 0 full K, 1 K < end of the row tile, 2 K >= start of the row tile. */
+int mq_gemm_f32(const float* A, long sam, long sak, const float* B, long sbk, long sbn, float* C, long ldc, int M,
+                int N, int K, float alpha, float beta, int tri, int ktrim, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOEQUANT_HIP_H */

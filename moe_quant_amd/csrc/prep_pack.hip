@@ -1,0 +1,246 @@
+// HBM-bound helpers around the column loop: group scales, transposed fp32 weights, code
+// transposition and int4 -> int32 packing.  All streaming kernels; lanes always run along the
+// contiguous dimension of whatever they read or write, transposes go through LDS.
+#include <hip/hip_fp16.h>
+
+#include "common.hpp"
+
+namespace {
+
+enum { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+
+__device__ __forceinline__ float load_as_f32(const void* p, long idx, int dt) {
+  if (dt == DT_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[idx]);
+  if (dt == DT_F16) return __half2float(reinterpret_cast<const __half*>(p)[idx]);
+  return reinterpret_cast<const float*>(p)[idx];
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Symmetric group scales: one wavefront per (row, group).
+//   scale = round_to(dtype)( (2/maxq as fp32) * max|w| + 1e-12 )
+// written compact (R,G) and, optionally, transposed (G,R) for the column loop.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void grid_sym_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C, int g,
+                                                       int G, const uint8_t* __restrict__ dead, float two_over_maxq,
+                                                       int round_dt, float* __restrict__ scale_rg,
+                                                       float* __restrict__ scale_gr) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)R * G) return;
+  const int row = (int)(item / G), grp = (int)(item - (long)row * G);
+  const int c0 = grp * g, c1 = min(C, c0 + g);
+  float m = 0.f;
+  for (int c = c0 + lane; c < c1; c += 64) {
+    float v = load_as_f32(W, (long)row * ldw + c, wdt);
+    if (dead && dead[c]) v = 0.f;
+    m = fmaxf(m, fabsf(v));
+  }
+  m = wave_max(m);
+  if (lane == 0) {
+    float s = two_over_maxq * m;
+    s = s + 1e-12f;
+    if (round_dt == DT_BF16) s = round_to_bf16(s);
+    if (round_dt == DT_F16) s = __half2float(__float2half_rn(s));
+    scale_rg[(long)row * G + grp] = s;
+    if (scale_gr) scale_gr[(long)grp * R + row] = s;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wt[j, r] = W[r, perm[j]] as fp32 (0 for dead columns).  64x64 tiles through LDS.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void prepare_wt_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C,
+                                                         const int* __restrict__ perm, const uint8_t* __restrict__ dead,
+                                                         float* __restrict__ Wt, long ldwt) {
+  __shared__ float t[64][65];
+  const int j0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int j = j0 + tx;
+  int src = -1;
+  if (j < C) {
+    src = perm ? perm[j] : j;
+    if (dead && dead[src]) src = -1;
+  }
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = r0 + rr;
+    float v = 0.f;
+    if (r < R && src >= 0) v = load_as_f32(W, (long)r * ldw + src, wdt);
+    t[rr][tx] = v;
+  }
+  __syncthreads();
+  for (int jj = ty; jj < 64; jj += 4) {
+    if (j0 + jj < C && r0 + tx < R) Wt[(long)(j0 + jj) * ldwt + r0 + tx] = t[tx][jj];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// codes[r, c] = Qt[perm_inv[c], r]  (u8), 64x64 tiles through LDS.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void untranspose_codes_kernel(const uint8_t* __restrict__ Qt, int R, int C,
+                                                                const int* __restrict__ perm_inv,
+                                                                uint8_t* __restrict__ codes, long ldc) {
+  __shared__ uint8_t t[64][68];
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int c = c0 + cc;
+    uint8_t v = 0;
+    if (c < C && r0 + tx < R) {
+      const int j = perm_inv ? perm_inv[c] : c;
+      v = Qt[(long)j * R + r0 + tx];
+    }
+    t[cc][tx] = v;
+  }
+  __syncthreads();
+  for (int rr = ty; rr < 64; rr += 4) {
+    if (r0 + rr < R && c0 + tx < C) codes[(long)(r0 + rr) * ldc + c0 + tx] = t[tx][rr];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// int4 -> int32: word[r, k] = sum_{i<8} ((codes[r, 8k+i] - zero + 8) & 15) << 4i ; columns past C pack as 0.
+// One thread reads 16 codes (one 16-byte load) and writes two words (one 8-byte store).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pack_int4_kernel(const uint8_t* __restrict__ codes, long ldc, int R, int C,
+                                                        const float* __restrict__ zero, int G, int g,
+                                                        int32_t* __restrict__ out, long ldo, int words, int vec_ok) {
+  const int pairs = (words + 1) / 2;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)R * pairs) return;
+  const int r = (int)(idx / pairs), p = (int)(idx - (long)r * pairs);
+  const int c0 = p * 16;
+  const uint8_t* src = codes + (long)r * ldc + c0;
+  uint8_t b[16];
+  if (vec_ok && c0 + 16 <= C) {
+    const uint4 v = *reinterpret_cast<const uint4*>(src);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) b[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) b[i] = (c0 + i < C) ? src[i] : 0;
+  }
+  uint32_t lo = 0, hi = 0;
+  if (zero == nullptr) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      lo |= (uint32_t)(b[i] & 15u) << (4 * i);
+      hi |= (uint32_t)(b[8 + i] & 15u) << (4 * i);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      uint32_t u = 0;
+      if (c0 + i < C) {
+        const int z = (int)zero[(long)r * G + (c0 + i) / g];
+        u = (uint32_t)((int)b[i] - z + 8) & 15u;
+      }
+      if (i < 8) lo |= u << (4 * i);
+      else hi |= u << (4 * (i - 8));
+    }
+  }
+  int32_t* dst = out + (long)r * ldo + 2 * p;
+  if (vec_ok && 2 * p + 1 < words) {
+    *reinterpret_cast<int2*>(dst) = make_int2((int)lo, (int)hi);
+  } else {
+    dst[0] = (int)lo;
+    if (2 * p + 1 < words) dst[1] = (int)hi;
+  }
+}
+
+// Packed words straight from the loop's transposed codes: word[r, k] from Qt[perm_inv[8k+i], r].
+// 64 rows x 64 columns per workgroup; reads are 64-byte runs along r, writes 8 words per row.
+__global__ __launch_bounds__(256) void pack_from_qt_kernel(const uint8_t* __restrict__ Qt, int R, int C,
+                                                           const int* __restrict__ perm_inv,
+                                                           int32_t* __restrict__ out, long ldo, int words) {
+  __shared__ uint8_t t[64][68];
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int c = c0 + cc;
+    uint8_t v = 0;
+    if (c < C && r0 + tx < R) {
+      const int j = perm_inv ? perm_inv[c] : c;
+      v = Qt[(long)j * R + r0 + tx] & 15u;
+    }
+    t[cc][tx] = v;
+  }
+  __syncthreads();
+  // 64 rows x 8 words = 512 words, two per thread
+  for (int it = threadIdx.x; it < 512; it += 256) {
+    const int rr = it >> 3, k = it & 7;
+    const int wk = (c0 >> 3) + k;
+    if (r0 + rr < R && wk < words) {
+      uint32_t w = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w |= (uint32_t)t[8 * k + i][rr] << (4 * i);
+      out[(long)(r0 + rr) * ldo + wk] = (int)w;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int mq_quant_grid_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size, int bits,
+                                 const uint8_t* dead_cols, int round_dtype, float* scale_rg, float* scale_gr,
+                                 void* stream) {
+  if (!W || !scale_rg || R <= 0 || C <= 0 || group_size <= 0 || C % group_size != 0) return MQ_ERR_ARG;
+  if (w_dtype < 0 || w_dtype > 2 || round_dtype < 0 || round_dtype > 2 || bits < 2 || bits > 8 || ldw < C)
+    return MQ_ERR_ARG;
+  const int G = C / group_size;
+  const float maxq = (float)((1 << bits) - 1);
+  const float two_over_maxq = 2.0f / maxq;
+  const long items = (long)R * G;
+  hipLaunchKernelGGL(grid_sym_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, W, w_dtype,
+                     ldw, R, C, group_size, G, dead_cols, two_over_maxq, round_dtype, scale_rg, scale_gr);
+  return mq_check_launch();
+}
+
+extern "C" int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int* perm,
+                             const uint8_t* dead_cols, float* Wt, long ldwt, void* stream) {
+  if (!W || !Wt || R <= 0 || C <= 0 || ldw < C || ldwt < R || w_dtype < 0 || w_dtype > 2) return MQ_ERR_ARG;
+  hipLaunchKernelGGL(prepare_wt_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream, W,
+                     w_dtype, ldw, R, C, perm, dead_cols, Wt, ldwt);
+  return mq_check_launch();
+}
+
+extern "C" int mq_untranspose_codes(const uint8_t* Qt, int R, int C, const int* perm_inv, uint8_t* codes, long ldc,
+                                    void* stream) {
+  if (!Qt || !codes || R <= 0 || C <= 0 || ldc < C) return MQ_ERR_ARG;
+  hipLaunchKernelGGL(untranspose_codes_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream,
+                     Qt, R, C, perm_inv, codes, ldc);
+  return mq_check_launch();
+}
+
+extern "C" int mq_pack_int4(const uint8_t* codes, long ldc, int R, int C, const float* zero, int group_size,
+                            int32_t* out, long ldo, void* stream) {
+  if (!codes || !out || R <= 0 || C <= 0 || ldc < C) return MQ_ERR_ARG;
+  const int words = (C + 7) / 8;
+  if (ldo < words) return MQ_ERR_ARG;
+  int G = 0;
+  if (zero) {
+    if (group_size <= 0 || C % group_size != 0) return MQ_ERR_ARG;
+    G = C / group_size;
+  }
+  const int vec_ok = ((uintptr_t)codes % 16 == 0) && (ldc % 16 == 0) && ((uintptr_t)out % 8 == 0) && (ldo % 2 == 0);
+  const long threads = (long)R * ((words + 1) / 2);
+  hipLaunchKernelGGL(pack_int4_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream, codes,
+                     ldc, R, C, zero, G, group_size, out, ldo, words, vec_ok);
+  return mq_check_launch();
+}
+
+extern "C" int mq_pack_from_qt(const uint8_t* Qt, int R, int C, const int* perm_inv, int32_t* out, long ldo,
+                               void* stream) {
+  if (!Qt || !out || R <= 0 || C <= 0) return MQ_ERR_ARG;
+  const int words = (C + 7) / 8;
+  if (ldo < words) return MQ_ERR_ARG;
+  hipLaunchKernelGGL(pack_from_qt_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream, Qt, R,
+                     C, perm_inv, out, ldo, words);
+  return mq_check_launch();
+}

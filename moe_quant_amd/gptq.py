@@ -1,0 +1,209 @@
+"""Drop-in for MoE-Quant's src/gptq.py: the same `GPTQ` handle, its numeric work done by HIP kernels.
+
+Out of scope (raise instead of silently differing): asymmetric grids, conv layers, the MSE scale
+search, the multi-GPU Hessian all-reduce.  Inputs to `update` must be bf16 (the engine's SYRK reads
+bf16 tokens directly; bf16 x bf16 products are exact in fp32, so nothing is lost versus the
+reference's up-cast to fp32)."""
+from __future__ import annotations
+
+import warnings
+from enum import Enum
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from . import linalg_utils, ops
+
+
+class QuantizationOrder(Enum):
+    DEFAULT = "default"
+    ACTIVATION = "activation"
+
+
+class GPTQ:
+    """Mirror of src/gptq.py:22-243 (constructor arguments, attributes and methods keep their names)."""
+
+    def __init__(
+        self,
+        layer: nn.Module,
+        group_size: Optional[int] = None,
+        sym: bool = False,
+        rel_damp: float = 1e-2,
+        block_size: int = None,
+        quantization_order: str = "default",
+        quantization_scale: str = "absmax",
+        is_distributed: bool = False,
+        tied_gptq_handle: Optional["GPTQ"] = None,
+    ):
+        self._validate_layer(layer)
+        self.layer = layer
+        self.W = self.layer.weight
+        self.d_row, self.d_col = layer.weight.shape[0], int(np.prod(layer.weight.shape[1:]))  # src/model_utils.py:11-12
+        self.sym = sym
+        self.group_size = group_size
+        self.rel_damp = rel_damp
+        self.block_size = block_size or self.d_col
+        self.quantization_order = QuantizationOrder(quantization_order)
+        self.quantization_scale = quantization_scale
+        if quantization_scale != "absmax":
+            # the reference compares this string with an Enum member, which never matches: absmax runs
+            warnings.warn(f"quantization_scale={quantization_scale!r} behaves as 'absmax', as in MoE-Quant")
+        self.W_device = self.W.device
+        self.W_dtype = self.W.dtype
+        self.W_shape = self.W.shape
+        self.H = None
+        self.num_samples = 0
+        self.is_distributed = is_distributed
+        self.tied_gptq_handle = tied_gptq_handle
+        self.num_tied_handles = 0
+        if tied_gptq_handle is not None:
+            tied_gptq_handle.num_tied_handles += 1
+        self.issue_zero_samples = False
+        self.issue_nan_hessian = False
+        self.issue_non_invertible = False
+        # engine state shared with tied handles (the reference recomputes both for every tied handle)
+        self._perm = None
+        self._hessian_inv = None
+
+    @staticmethod
+    def _validate_layer(layer):
+        assert isinstance(layer, nn.Linear), "this engine supports nn.Linear layers only"
+
+    def has_hessian_issues(self) -> bool:
+        return any([self.issue_zero_samples, self.issue_nan_hessian, self.issue_non_invertible])
+
+    # ---- Hessian accumulation: src/gptq.py:73-105 ---------------------------------------------------
+    @torch.no_grad()
+    def update(self, input: Tensor) -> None:
+        if self.H is None:
+            self.H = torch.zeros((self.d_col, self.d_col), device=input.device, dtype=torch.float32)
+        input = input.reshape(-1, input.shape[-1])
+        if input.dtype != torch.bfloat16:
+            raise TypeError(f"GPTQ.update needs bf16 activations, got {input.dtype}")
+        num_new_samples = input.shape[0]
+        if num_new_samples == 0:
+            return  # the reference would divide 0/0 here when nothing was collected before
+        beta = self.num_samples / (self.num_samples + num_new_samples)
+        alpha = 2.0 / (self.num_samples + num_new_samples)
+        ops.hessian_syrk_(self.H, input, beta, alpha, mirror=True)
+        self.num_samples += num_new_samples
+
+    add_batch = update
+
+    @property
+    def tokens_collected(self) -> int:
+        return self.num_samples
+
+    def reset(self) -> None:
+        """src/gptq.py:111-120."""
+        self.W = self.layer.weight
+        if self.num_tied_handles == 0:
+            self.H = None
+            self._hessian_inv = None
+        elif self.tied_gptq_handle:
+            self.tied_gptq_handle.num_tied_handles -= 1
+            if self.tied_gptq_handle.num_tied_handles == 0:
+                self.tied_gptq_handle.H = None
+                self.tied_gptq_handle._hessian_inv = None
+        self.num_samples = 0
+        self._perm = None
+        if self.tied_gptq_handle is not None:
+            self._hessian_inv = None
+        torch.cuda.empty_cache()
+
+    # ---- pre-step: src/gptq.py:122-154 --------------------------------------------------------------
+    @torch.no_grad()
+    def quantization_pre_step(self) -> None:
+        if self.H is None:
+            if self.tied_gptq_handle:
+                self.H = self.tied_gptq_handle.H
+            else:
+                self.H = torch.eye(self.d_col, device=self.W_device, dtype=torch.float32)
+                self.issue_zero_samples = True
+        if self.is_distributed and torch.distributed.is_available() and torch.distributed.is_initialized():
+            if torch.distributed.get_world_size() > 1:
+                raise NotImplementedError("the multi-GPU Hessian all-reduce is outside this engine's scope")
+        if torch.isnan(self.H).any().item():
+            self.H = torch.eye(self.d_col, device=self.W_device, dtype=torch.float32)
+            self.issue_nan_hessian = True
+        pruned_ids = torch.diag(self.H) == 0
+        self.H[pruned_ids, pruned_ids] = 1
+        self.W = self.W.clone().float()
+        self.W[:, pruned_ids] = 0
+        self.pre_step_completed = True
+
+    # ---- quantize: src/gptq.py:156-218 ---------------------------------------------------------------
+    @torch.no_grad()
+    def _quantize(self, bits: int) -> Tuple[Tensor, Tensor, Tensor]:
+        if not self.sym:
+            raise NotImplementedError("only symmetric quantization is supported (as MoE-Quant's README states)")
+        d_col, dtype, device = self.d_col, self.W_dtype, self.W_device
+        group_size = self.group_size or d_col
+        W = self.W
+        # per-group scales from the un-updated weights (src/gptq.py:171-178): compact (R,G) and (G,R)
+        scale_rg, scale_gr = ops.quant_grid_sym(W, group_size, bits, dtype)
+        tied = self.tied_gptq_handle
+        perm = perm_inv = perm_i32 = perm_inv_i32 = None
+        if self.quantization_order == QuantizationOrder.ACTIVATION:
+            if tied is not None and tied._perm is not None:
+                # the owner's H is already permuted; reuse its order (the reference re-sorts the sorted
+                # diagonal here, gets the identity and pairs un-permuted weights with a permuted H)
+                perm = tied._perm
+            else:
+                perm = torch.argsort(self.H.diag(), descending=True)
+            perm_inv = torch.argsort(perm)
+            perm_i32, perm_inv_i32 = perm.to(torch.int32), perm_inv.to(torch.int32)
+            self._perm = perm
+            if tied is None:
+                self.H = self.H[perm][:, perm]
+        hessian_inv = self._get_hessian_inverse()
+        Wt = ops.prepare_wt(W, perm_i32)
+        if perm is None:
+            scale_row = torch.arange(d_col, device=device, dtype=torch.int32) // group_size
+        else:
+            scale_row = (perm // group_size).to(torch.int32)
+        maxq = float(2**bits - 1)
+        qzero = float(2 ** (bits - 1))
+        Qt = ops.gptq_loop_(Wt, hessian_inv, scale_gr, scale_row, None, qzero, maxq, dtype, self.block_size)
+        self._Qt, self._perm_inv_i32 = Qt, perm_inv_i32
+        qweight = ops.untranspose_codes(Qt, perm_inv_i32)
+        scale = scale_rg.to(dtype)
+        zero = torch.full_like(scale, qzero)
+        return qweight, scale, zero
+
+    def quantize(self, bits: int | float) -> Tuple[Tensor, Tensor, Tensor]:
+        self.quantization_pre_step()
+        return self._quantize(bits)
+
+    def packed_words(self) -> Tensor:
+        """int32 (R, C/8) compressed_tensors words of the last `quantize` call, packed straight from the
+        loop's own code buffer (same bits as pack_weight on the returned qweight)."""
+        return ops.pack_from_qt(self._Qt, self._perm_inv_i32)
+
+    # ---- inverse factor: src/gptq.py:220-243 ---------------------------------------------------------
+    @torch.no_grad()
+    def _get_hessian_inverse(self) -> Tensor:
+        tied = self.tied_gptq_handle
+        if tied is not None and tied._hessian_inv is not None and tied.H is self.H:
+            return tied._hessian_inv  # same damped H -> same factor; the reference recomputes it
+        w = self.W
+        zero_cols = torch.nonzero(w.eq(0).all(dim=0))
+        H = self.H
+        if not tied:
+            H[zero_cols, :] = 0
+            H[:, zero_cols] = 0
+            H[zero_cols, zero_cols] = 1
+            damp = self.rel_damp * torch.diag(self.H).mean()
+            self.H.diagonal().add_(damp)
+        U, info = linalg_utils.inverse_cholesky_factor(H)
+        if int(info.item()) != 0:
+            # the reference's bare `except` around cholesky lands here (src/gptq.py:239-240); it never sets
+            # issue_non_invertible, this engine does
+            self.issue_non_invertible = True
+            U = torch.eye(self.d_col, device=H.device, dtype=torch.float32)
+        if self.num_tied_handles > 0:
+            self._hessian_inv = U
+        return U

@@ -1,0 +1,197 @@
+"""Tensor-level wrappers over the C ABI.  torch is used for device memory and the current stream only;
+every computation below happens in libmoequant_hip.so."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import DT_BF16, DT_F16, DT_F32, check
+
+_DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
+
+
+def _dt(dtype: Optional[torch.dtype]) -> int:
+    if dtype is None:
+        return DT_F32
+    if dtype not in _DT:
+        raise TypeError(f"unsupported dtype {dtype}")
+    return _DT[dtype]
+
+
+def _stream(t: Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _dev(*ts: Optional[Tensor]) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise _lib.MoeQuantHipError("moe_quant_amd kernels need GPU tensors; there is no CPU path")
+
+
+def _p(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+class _Workspace:
+    """One growing scratch buffer per device so the hot path does not hit the allocator."""
+
+    def __init__(self):
+        self.buf = {}
+
+    def get(self, device: torch.device, nbytes: int) -> Tensor:
+        key = (device.type, device.index)
+        b = self.buf.get(key)
+        if b is None or b.numel() < nbytes:
+            b = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+            self.buf[key] = b
+        return b
+
+
+_ws = _Workspace()
+
+
+# ---- (1) Hessian ------------------------------------------------------------------------------------
+def hessian_syrk_(H: Tensor, X: Tensor, beta: float, alpha: float, mirror: bool = True) -> Tensor:
+    """H <- beta*H + alpha*X^T X in place.  H (C,C) fp32, X (n,C) bf16, rows may be strided."""
+    _dev(H, X)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    if X.dtype != torch.bfloat16 or X.dim() != 2 or X.shape[1] != C:
+        raise ValueError("X must be (n,C) bf16")
+    if X.shape[0] > 0 and X.stride(1) != 1:
+        X = X.contiguous()
+    n = X.shape[0]
+    need = lib.mq_hessian_syrk_workspace_bytes(n, C)
+    ws = _ws.get(H.device, need) if need else None
+    ldx = X.stride(0) if n > 1 else C
+    rc = lib.mq_hessian_syrk_bf16(
+        H.data_ptr(), H.stride(0), X.data_ptr() if n else None, ldx, n, C, beta, alpha, int(mirror),
+        _p(ws), need, _stream(H),
+    )
+    check(rc, "mq_hessian_syrk_bf16")
+    return H
+
+
+# ---- (2) factorisation -------------------------------------------------------------------------------
+def factor_upper_inverse_(A: Tensor, info: Optional[Tensor] = None, normalize: bool = True) -> Tensor:
+    """In place A -> upper U = chol(A^-1, upper), rows scaled to unit diagonal when `normalize`.
+    Returns the device int32 `info` (0 = success)."""
+    _dev(A, info)
+    lib = _lib.load()
+    C = A.shape[0]
+    if A.dtype != torch.float32 or A.shape != (C, C) or A.stride(1) != 1 or C % 128:
+        raise ValueError("A must be (C,C) fp32, unit column stride, C % 128 == 0")
+    if info is None:
+        info = torch.zeros(1, dtype=torch.int32, device=A.device)
+    rc = lib.mq_factor_upper_inverse(A.data_ptr(), A.stride(0), C, int(normalize), info.data_ptr(), _stream(A))
+    check(rc, "mq_factor_upper_inverse")
+    return info
+
+
+# ---- (3) grid, layout, loop --------------------------------------------------------------------------
+def quant_grid_sym(W: Tensor, group_size: int, bits: int, round_dtype, dead_cols: Optional[Tensor] = None,
+                   want_transposed: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
+    _dev(W, dead_cols)
+    lib = _lib.load()
+    R, C = W.shape
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    G = C // group_size
+    s_rg = torch.empty(R, G, dtype=torch.float32, device=W.device)
+    s_gr = torch.empty(G, R, dtype=torch.float32, device=W.device) if want_transposed else None
+    rc = lib.mq_quant_grid_sym(W.data_ptr(), _dt(W.dtype), W.stride(0), R, C, group_size, bits, _p(dead_cols),
+                               _dt(round_dtype), s_rg.data_ptr(), _p(s_gr), _stream(W))
+    check(rc, "mq_quant_grid_sym")
+    return s_rg, s_gr
+
+
+def prepare_wt(W: Tensor, perm: Optional[Tensor] = None, dead_cols: Optional[Tensor] = None) -> Tensor:
+    _dev(W, perm, dead_cols)
+    lib = _lib.load()
+    R, C = W.shape
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    Wt = torch.empty(C, R, dtype=torch.float32, device=W.device)
+    rc = lib.mq_prepare_wt(W.data_ptr(), _dt(W.dtype), W.stride(0), R, C, _p(perm), _p(dead_cols), Wt.data_ptr(), R,
+                           _stream(W))
+    check(rc, "mq_prepare_wt")
+    return Wt
+
+
+def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor], qzero: Optional[Tensor],
+               qzero_const: float, maxq: float, round_dtype, block: int) -> Tensor:
+    """Runs the loop in place on Wt (C,R); returns the codes Qt (C,R) uint8."""
+    _dev(Wt, U, scale, scale_row, qzero)
+    lib = _lib.load()
+    C, R = Wt.shape
+    for t in (Wt, U, scale) + ((qzero,) if qzero is not None else ()):
+        if t.dtype != torch.float32 or t.stride(-1) != 1:
+            raise ValueError("Wt, U, scale, qzero must be fp32 with unit inner stride")
+    if qzero is not None and (qzero.shape != scale.shape or qzero.stride(0) != scale.stride(0)):
+        raise ValueError("qzero must have the layout of scale")
+    if scale_row is not None and (scale_row.dtype != torch.int32 or scale_row.numel() != C):
+        raise ValueError("scale_row must be int32 of length C")
+    if scale_row is None and scale.shape[0] != C:
+        raise ValueError("scale must be (C,R) when no scale_row map is given")
+    Qt = torch.empty(C, R, dtype=torch.uint8, device=Wt.device)
+    E = _ws.get(Wt.device, 128 * R * 4)
+    rc = lib.mq_gptq_loop(Wt.data_ptr(), Wt.stride(0), C, R, U.data_ptr(), U.stride(0), scale.data_ptr(),
+                          scale.stride(0), _p(scale_row), _p(qzero), qzero_const, maxq, _dt(round_dtype), block,
+                          Qt.data_ptr(), E.data_ptr(), _stream(Wt))
+    check(rc, "mq_gptq_loop")
+    return Qt
+
+
+def untranspose_codes(Qt: Tensor, perm_inv: Optional[Tensor] = None) -> Tensor:
+    _dev(Qt, perm_inv)
+    lib = _lib.load()
+    C, R = Qt.shape
+    codes = torch.empty(R, C, dtype=torch.uint8, device=Qt.device)
+    rc = lib.mq_untranspose_codes(Qt.data_ptr(), R, C, _p(perm_inv), codes.data_ptr(), C, _stream(Qt))
+    check(rc, "mq_untranspose_codes")
+    return codes
+
+
+# ---- (4) packing -------------------------------------------------------------------------------------
+def pack_int4(codes: Tensor, zero: Optional[Tensor] = None, group_size: int = 0) -> Tensor:
+    """codes (R,C) uint8 -> (R, ceil(C/8)) int32; zero (R,G) fp32 or None (= 8)."""
+    _dev(codes, zero)
+    lib = _lib.load()
+    if codes.dtype != torch.uint8 or codes.dim() != 2:
+        raise ValueError("codes must be (R,C) uint8")
+    if codes.stride(1) != 1:
+        codes = codes.contiguous()
+    R, C = codes.shape
+    words = (C + 7) // 8
+    out = torch.empty(R, words, dtype=torch.int32, device=codes.device)
+    if zero is not None:
+        zero = zero.to(torch.float32).contiguous()
+    rc = lib.mq_pack_int4(codes.data_ptr(), codes.stride(0), R, C, _p(zero), group_size, out.data_ptr(), words,
+                          _stream(codes))
+    check(rc, "mq_pack_int4")
+    return out
+
+
+def pack_from_qt(Qt: Tensor, perm_inv: Optional[Tensor] = None) -> Tensor:
+    _dev(Qt, perm_inv)
+    lib = _lib.load()
+    C, R = Qt.shape
+    words = (C + 7) // 8
+    out = torch.empty(R, words, dtype=torch.int32, device=Qt.device)
+    rc = lib.mq_pack_from_qt(Qt.data_ptr(), R, C, _p(perm_inv), out.data_ptr(), words, _stream(Qt))
+    check(rc, "mq_pack_from_qt")
+    return out
+
+
+def gemm_f32_(A, sam, sak, B, sbk, sbn, Cm, M, N, K, alpha=1.0, beta=0.0, tri=0, ktrim=0):
+    _dev(A, B, Cm)
+    lib = _lib.load()
+    rc = lib.mq_gemm_f32(A.data_ptr(), sam, sak, B.data_ptr(), sbk, sbn, Cm.data_ptr(), Cm.stride(0), M, N, K, alpha,
+                         beta, tri, ktrim, _stream(Cm))
+    check(rc, "mq_gemm_f32")
+    return Cm

@@ -1,0 +1,99 @@
+"""Drop-in for the hot-path part of MoE-Quant's src/quant_utils.py.
+
+get_quantization_grid (absmax, symmetric) runs on the HIP grid kernel; the small elementwise helpers
+(quantize / dequantize / round_fp / dequantize_linear_weight / get_relative_mse_error) are the
+reference's own torch one-liners and stay torch: they are metrics and test helpers, not the path."""
+from __future__ import annotations
+
+import warnings
+from enum import Enum
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import ops
+
+
+class QuantizationScale(Enum):
+    ABSMAX = "absmax"
+    MSE = "mse"
+
+
+def round_fp(x: Tensor, dtype: torch.dtype = None) -> Tensor:
+    """src/quant_utils.py:52-53."""
+    return x if dtype is None else x.to(dtype=dtype).to(x.dtype)
+
+
+def quantize(x: Tensor, scale: Tensor, qzero: Tensor, maxq: Tensor) -> Tensor:
+    """src/quant_utils.py:57-58 (round-half-even torch helper)."""
+    return (x / scale + qzero).round().clamp(torch.zeros_like(maxq), maxq)
+
+
+def dequantize(qx: Tensor, scale: Tensor, qzero: Tensor, dtype: torch.dtype = None) -> Tensor:
+    """src/quant_utils.py:61-62."""
+    return round_fp((qx - qzero) * scale, dtype)
+
+
+def dequantize_quantized(x, scale, qzero, maxq, dtype=None):
+    """src/quant_utils.py:65-68."""
+    return dequantize(quantize(x, scale, qzero, maxq), scale, qzero, dtype)
+
+
+def find_quantization_meta(x: Tensor, bit_width: int, symmetric: bool = False, dtype: torch.dtype = None):
+    """src/quant_utils.py:75-101 for x of shape (..., G, g): per-group scale, qzero, maxq.  Symmetric only."""
+    if not symmetric:
+        raise NotImplementedError("only symmetric quantization is supported (as MoE-Quant's README states)")
+    *lead, G, g = x.shape
+    x2 = x.reshape(-1, G * g)
+    scale, _ = ops.quant_grid_sym(x2, g, bit_width, dtype, want_transposed=False)
+    maxq = torch.tensor(2**bit_width - 1, dtype=x.dtype, device=x.device)
+    scale = scale.to(x.dtype).reshape(*lead, G)
+    qzero = torch.full_like(scale, (2**bit_width) * 0.5)
+    return scale, qzero, maxq
+
+
+@torch.no_grad()
+def get_quantization_grid(
+    weight: Tensor,
+    group_size: int,
+    bits: int,
+    symmetric: bool = False,
+    dtype: torch.dtype = None,
+    quantization_scale=QuantizationScale.ABSMAX,
+    quant_max_shrink: float = 0.2,
+    quant_n_grid: int = 100,
+    quant_norm: float = 2.4,
+):
+    """src/quant_utils.py:195-240: returns (scale (...,C), qzero (...,C), maxq ()) replicated per column."""
+    if quantization_scale == QuantizationScale.MSE:
+        raise NotImplementedError("MSE scale search is outside this engine's scope")
+    if isinstance(quantization_scale, str) and quantization_scale != "absmax":
+        # the reference compares this string to an Enum, which is never equal: absmax is what it runs
+        warnings.warn(f"quantization_scale={quantization_scale!r} behaves as 'absmax', as in MoE-Quant")
+    group_size = group_size or weight.shape[-1]
+    w = weight.unflatten(dim=-1, sizes=(-1, group_size))
+    scale, qzero, maxq = find_quantization_meta(w, bits, symmetric, dtype)
+    scale = scale.repeat_interleave(group_size, dim=-1)
+    qzero = qzero.repeat_interleave(group_size, dim=-1)
+    assert weight.shape == scale.shape == qzero.shape and maxq.shape == ()
+    return scale, qzero, maxq
+
+
+def dequantize_linear_weight(qweight: Tensor, scale: Tensor, zero: Tensor, perm: Optional[Tensor] = None):
+    """src/quant_utils.py:243-256."""
+    scale = scale.view(qweight.shape[0], -1, 1)
+    zero = zero.view(qweight.shape[0], -1, 1)
+    num_groups = scale.shape[1]
+    weight = dequantize(qweight.view(qweight.shape[0], num_groups, -1), scale, zero).view_as(qweight)
+    if perm is not None:
+        weight = weight[:, perm.argsort()]
+    return weight
+
+
+def get_relative_mse_error(q: Tensor, w: Tensor, H: Optional[Tensor] = None):
+    """src/quant_utils.py:259-264."""
+    delta = q - w
+    if H is None:
+        return delta.pow(2).mean() / w.pow(2).mean()
+    return delta.mm(H).mul(delta).mean() / (w.mm(H).mul(w).mean() + 1e-6)

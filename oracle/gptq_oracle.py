@@ -1,0 +1,343 @@
+"""CPU restatement of MoE-Quant's GPTQ hot path (torch, fp32 unless stated).
+
+THIS FILE IS TEST INFRASTRUCTURE.  It is the checker that the HIP kernels are
+compared against and the "reference torch CPU path" that bench.py times as the
+CPU baseline.  Nothing in the shipped package imports it; only tests/,
+__graft_entry__.smoke() and bench.py's cpu_baseline leg may.
+
+Every function cites the reference lines (relative to the MoE-Quant tree) that
+it follows.  The reference has no tests or golden vectors, so each function is
+pinned by closed forms / invariants / brute force in tests/test_oracle_*.py:
+
+  hessian_update ............ closed form (2/N) sum X^T X in fp64, batch-split invariance
+  quantization_pre_step ..... special cases (no samples, NaN, dead channel)
+  find_quantization_meta .... known answers (absmax 0.15 -> bf16(0.02), zero group -> bf16(1e-12))
+  act_order_perm ............ argsort of distinct values is unique; perm_inv[perm] == arange
+  hessian_inverse ........... torch's own LAPACK routines ARE the reference arithmetic; invariants
+                              (upper, unit diagonal, (DU)^T(DU) H = I), diagonal H, 2x2 by hand
+  gptq_loop ................. U = I -> plain round-to-nearest; fp64 un-blocked textbook GPTQ on tiny
+                              shapes; block-size invariance; row independence; C % B != 0
+  pack_int4 ................. closed form; known answer from upstream docstring ([1,2]@8bit -> 33409);
+                              round trip.  compressed_tensors is absent from this image and un-pinned
+                              by the reference (no version, no tests) -> "parity unpinned" beyond that.
+  dequantize / relative_mse . closed form; tr(dH d^T) = (2/n)||X d^T||_F^2 against fp64 matmul
+
+Unpinnable by any means: torch.argsort tie order (unstable sort) and the exact
+bits of Triton's fma / division on a GPU.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+# ----------------------------------------------------------------------------------------------
+# (a2) Hessian accumulation -- src/gptq.py:73-105
+# ----------------------------------------------------------------------------------------------
+
+
+def hessian_update(H: Optional[Tensor], num_samples: int, x: Tensor) -> Tuple[Tensor, int]:
+    """H <- n0/(n0+n) H + 2/(n0+n) X^T X in fp32 (src/gptq.py:82-105)."""
+    x = x.reshape(-1, x.shape[-1])  # src/gptq.py:86
+    if H is None:
+        H = torch.zeros((x.shape[-1], x.shape[-1]), dtype=torch.float32)  # src/gptq.py:82-83
+    x = x.float()  # src/gptq.py:97
+    n = x.shape[0]  # src/gptq.py:99
+    beta = num_samples / (num_samples + n)  # src/gptq.py:101
+    alpha = 2.0 / (num_samples + n)  # src/gptq.py:102
+    H.addmm_(x.T, x, beta=beta, alpha=alpha)  # src/gptq.py:103
+    return H, num_samples + n  # src/gptq.py:105
+
+
+def hessian_fp64(batches) -> Tensor:
+    """Ground truth (2/N) sum_b X_b^T X_b in float64 -- the 1e-5 Frobenius target."""
+    acc, n = None, 0
+    for x in batches:
+        x = x.reshape(-1, x.shape[-1]).double()
+        acc = x.T @ x if acc is None else acc + x.T @ x
+        n += x.shape[0]
+    return acc * (2.0 / n)
+
+
+# ----------------------------------------------------------------------------------------------
+# (a3) pre-step -- src/gptq.py:122-154
+# ----------------------------------------------------------------------------------------------
+
+
+def quantization_pre_step(H: Optional[Tensor], W: Tensor):
+    """Returns (H, W32, issue_zero_samples, issue_nan_hessian) -- src/gptq.py:129-152 (untied, single process)."""
+    d_col = W.shape[1]
+    zero_samples = nan_hessian = False
+    if H is None:  # src/gptq.py:129-134
+        H = torch.eye(d_col, dtype=torch.float32)
+        zero_samples = True
+    if torch.isnan(H).any().item():  # src/gptq.py:141-143
+        H = torch.eye(d_col, dtype=torch.float32)
+        nan_hessian = True
+    pruned = torch.diag(H) == 0  # src/gptq.py:145
+    H[pruned, pruned] = 1  # src/gptq.py:146
+    W = W.clone().float()  # src/gptq.py:149
+    W[:, pruned] = 0  # src/gptq.py:152
+    return H, W, zero_samples, nan_hessian
+
+
+# ----------------------------------------------------------------------------------------------
+# (a4) quantization grid -- src/quant_utils.py:52-101,195-240
+# ----------------------------------------------------------------------------------------------
+
+
+def round_fp(x: Tensor, dtype: Optional[torch.dtype]) -> Tensor:
+    """src/quant_utils.py:52-53."""
+    return x if dtype is None else x.to(dtype).to(x.dtype)
+
+
+def find_quantization_meta(x: Tensor, bit_width: int, dtype: Optional[torch.dtype]):
+    """Symmetric branch of src/quant_utils.py:75-96: reduction over the last dim."""
+    maxq = torch.tensor(2**bit_width - 1, dtype=x.dtype)  # :87
+    hi = x.amax(dim=-1)  # :89 (named x_min there; only |.| is used in the symmetric branch)
+    lo = x.amin(dim=-1)  # :90
+    scale = (2.0 / maxq) * torch.maximum(hi.abs(), lo.abs())  # :93
+    scale = round_fp(scale + 1e-12, dtype)  # :94
+    qzero = torch.full_like(scale, ((maxq + 1.0) * 0.5).item())  # :95
+    return scale, qzero, maxq
+
+
+def quantization_grid(W: Tensor, group_size: Optional[int], bits: int, dtype: Optional[torch.dtype]):
+    """Compact grid: scale (R,G) fp32 (bf16-exact), qzero (R,G), maxq () -- src/quant_utils.py:213-220."""
+    g = group_size or W.shape[-1]
+    return find_quantization_meta(W.unflatten(-1, (-1, g)), bits, dtype)
+
+
+def replicate_grid(scale: Tensor, qzero: Tensor, group_size: int):
+    """(R,G) -> (R,C) as src/quant_utils.py:234-235."""
+    return scale.repeat_interleave(group_size, dim=-1), qzero.repeat_interleave(group_size, dim=-1)
+
+
+def quantize(x: Tensor, scale: Tensor, qzero: Tensor, maxq: Tensor, half_up: bool = True) -> Tensor:
+    """half_up=True follows the Triton kernel used inside the loop (src/quant_utils.py:30-44:
+    floor(x/s + z + 0.5)); half_up=False follows the torch helper (:57-58, round-half-even).
+    The two differ only on exact ties."""
+    v = x / scale + qzero
+    r = torch.floor(v + 0.5) if half_up else v.round()
+    return r.clamp(torch.zeros_like(maxq), maxq)
+
+
+def dequantize(q: Tensor, scale: Tensor, qzero: Tensor, dtype: Optional[torch.dtype] = None) -> Tensor:
+    """src/quant_utils.py:61-62 / :47-49."""
+    return round_fp((q - qzero) * scale, dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# (a5) act-order -- src/gptq.py:179-187
+# ----------------------------------------------------------------------------------------------
+
+
+def act_order_perm(H: Tensor, act_order: bool):
+    if act_order:
+        perm = torch.argsort(H.diag(), descending=True)  # src/gptq.py:181
+    else:
+        perm = torch.arange(H.shape[0])  # src/gptq.py:183
+    return perm, torch.argsort(perm)  # src/gptq.py:184
+
+
+# ----------------------------------------------------------------------------------------------
+# (a6) damped inverse factor -- src/gptq.py:220-243, src/linalg_utils.py:8-12
+# ----------------------------------------------------------------------------------------------
+
+
+def hessian_inverse(H: Tensor, W: Tensor, rel_damp: float, dtype=torch.float32):
+    """H is modified in place (masking + damping) exactly as the reference does; returns
+    (U, ok) with U = unit-diagonal upper factor; ok=False means the identity fallback fired.
+    `dtype=torch.float64` gives the high-precision truth used to bound factorisation error."""
+    d_col = H.shape[0]
+    zero_cols = torch.nonzero(W.eq(0).all(dim=0))  # src/gptq.py:224
+    H[zero_cols, :] = 0  # :228
+    H[:, zero_cols] = 0  # :229
+    H[zero_cols, zero_cols] = 1  # :230
+    damp = rel_damp * torch.diag(H).mean()  # :233
+    H[range(d_col), range(d_col)] += damp  # :234
+    ok = True
+    try:
+        Hi = torch.cholesky_inverse(torch.linalg.cholesky(H.to(dtype)))  # src/linalg_utils.py:12
+        U = torch.linalg.cholesky(Hi, upper=True)  # src/gptq.py:238
+    except Exception:  # bare except at src/gptq.py:239
+        U = torch.eye(d_col, dtype=dtype)
+        ok = False
+    U.div_(U.diag()[:, None])  # src/gptq.py:242
+    return U, ok
+
+
+# ----------------------------------------------------------------------------------------------
+# (a7-a10) the blocked loop -- src/gptq_loop.py:141-148 with kernel bodies :28-40 and :77-88
+# ----------------------------------------------------------------------------------------------
+
+
+def _fma32(a: Tensor, b: Tensor, c: Tensor) -> Tensor:
+    """fp32 fused multiply-add (tl.fma, src/gptq_loop.py:86): the fp32*fp32 product is exact in
+    fp64; one fp64 add then one fp32 rounding (double rounding is possible only on ~2^-29 ties)."""
+    return (a.double() * b.double() + c.double()).float()
+
+
+def gptq_loop(
+    weight: Tensor,
+    hessian_inv: Tensor,
+    scale: Tensor,
+    qzero: Tensor,
+    maxq: Tensor,
+    dtype: Optional[torch.dtype],
+    gptq_block_size: int = 128,
+    half_up: bool = True,
+    fused: bool = True,
+) -> Tensor:
+    """weight (C,R) fp32 is modified in place to the dequantized values; returns codes (C,R) fp32.
+    Mirrors gptq_loop_graph(direct=True), src/gptq_loop.py:141-148."""
+    C, R = weight.shape
+    if gptq_block_size <= 0:  # src/gptq_loop.py:212-213
+        gptq_block_size = C
+    qweight = torch.empty_like(weight)
+    err = torch.empty(gptq_block_size, R, dtype=weight.dtype)
+    for i1 in range(0, C, gptq_block_size):
+        i2 = min(i1 + gptq_block_size, C)
+        for j in range(i1, i2):
+            x = weight[j]
+            q = quantize(x, scale[j], qzero[j], maxq, half_up)  # tl_quantize, src/gptq_loop.py:34
+            y = dequantize(q, scale[j], qzero[j], dtype)  # tl_dequantize, :35
+            e = y - x  # :36
+            weight[j] = y  # :38
+            qweight[j] = q  # :39
+            err[j - i1] = e  # :40
+            if j + 1 < i2:  # addvv: C[a,:] = fma(va[a], vb[:], C[a,:]), :77-88
+                h = hessian_inv[j, j + 1 : i2, None]
+                if fused:
+                    weight[j + 1 : i2] = _fma32(h, e[None, :], weight[j + 1 : i2])
+                else:
+                    weight[j + 1 : i2] += h * e[None, :]
+        if i2 < C:
+            weight[i2:].addmm_(hessian_inv[i1:i2, i2:].t(), err[: i2 - i1], beta=1, alpha=1)  # :148
+    return qweight
+
+
+# ----------------------------------------------------------------------------------------------
+# whole linear: GPTQ.quantize -- src/gptq.py:156-218
+# ----------------------------------------------------------------------------------------------
+
+
+def quantize_linear(
+    W: Tensor,
+    H: Optional[Tensor],
+    bits: int = 4,
+    group_size: Optional[int] = 128,
+    rel_damp: float = 1e-2,
+    block_size: Optional[int] = 128,
+    act_order: bool = False,
+    dtype: Optional[torch.dtype] = None,
+    half_up: bool = True,
+    inverse_dtype=torch.float32,
+):
+    """Returns dict(qweight u8 (R,C), scale (R,G), zero (R,G), U, perm, H (damped, permuted), ok)."""
+    dtype = dtype or W.dtype
+    R, C = W.shape
+    H, W32, zero_samples, nan_h = quantization_pre_step(H, W)
+    g = group_size or C
+    scale_g, zero_g, maxq = quantization_grid(W32, g, bits, dtype)  # src/gptq.py:171-178
+    scale, zero = replicate_grid(scale_g, zero_g, g)
+    perm, perm_inv = act_order_perm(H, act_order)
+    H = H[perm][:, perm]  # src/gptq.py:187
+    U, ok = hessian_inverse(H, W32, rel_damp, inverse_dtype)  # :189
+    U = U.float()
+    Wt = W32.t()[perm].contiguous()  # :192
+    q = gptq_loop(
+        Wt,
+        U,
+        scale.t()[perm].contiguous(),
+        zero.t()[perm].contiguous(),
+        maxq,
+        dtype,
+        block_size or C,
+        half_up,
+    )
+    qweight = q[perm_inv].t().contiguous().to(torch.uint8)  # :199
+    return dict(
+        qweight=qweight,
+        scale=scale[:, ::g].to(dtype),  # :201
+        zero=zero[:, ::g].to(dtype),  # :202
+        U=U,
+        perm=perm,
+        H=H,
+        ok=ok,
+        issue_zero_samples=zero_samples,
+        issue_nan_hessian=nan_h,
+    )
+
+
+# ----------------------------------------------------------------------------------------------
+# (a12-a13) dequantize + error metric -- src/quant_utils.py:243-264
+# ----------------------------------------------------------------------------------------------
+
+
+def dequantize_linear_weight(qweight: Tensor, scale: Tensor, zero: Tensor, perm: Optional[Tensor] = None) -> Tensor:
+    R = qweight.shape[0]
+    s = scale.view(R, -1, 1)
+    z = zero.view(R, -1, 1)
+    w = dequantize(qweight.view(R, s.shape[1], -1), s, z).view_as(qweight)  # :250 (u8 - bf16 -> bf16)
+    if perm is not None:
+        w = w[:, perm.argsort()]  # :253-255
+    return w
+
+
+def relative_mse(q: Tensor, w: Tensor, H: Optional[Tensor] = None) -> Tensor:
+    d = q - w
+    if H is None:
+        return d.pow(2).mean() / w.pow(2).mean()  # :262
+    return d.mm(H).mul(d).mean() / (w.mm(H).mul(w).mean() + 1e-6)  # :264
+
+
+# ----------------------------------------------------------------------------------------------
+# (a14) packing -- pack_quantized_model.py:57-75 + compressed_tensors.pack_to_int32 (absent here)
+# ----------------------------------------------------------------------------------------------
+
+
+def pack_to_int32(value: Tensor, num_bits: int) -> Tensor:
+    """Published algorithm of compressed_tensors.compressors.pack_to_int32 (no version pinned by the
+    reference, package absent from this image): int8 input, offset by 2^(bits-1) to unsigned,
+    pad the last dim to a multiple of 32/bits, element i of each word in bits [bits*i, bits*i+bits)."""
+    if value.dtype != torch.int8:
+        raise ValueError("Tensor must be quantized to torch.int8 before packing")
+    if num_bits > 8:
+        raise ValueError("Packing is only supported for less than 8 bits")
+    u = (value.to(torch.int16) + (1 << (num_bits - 1))).to(torch.int64) & ((1 << num_bits) - 1)
+    pf = 32 // num_bits
+    rows, cols = u.shape
+    pad = (-cols) % pf
+    if pad:
+        u = torch.nn.functional.pad(u, (0, pad))
+    u = u.view(rows, -1, pf)
+    shifts = torch.arange(pf, dtype=torch.int64) * num_bits
+    word = (u << shifts).sum(-1)  # disjoint bit fields: sum == or
+    word = torch.where(word >= 2**31, word - 2**32, word)
+    return word.to(torch.int32)
+
+
+def unpack_from_int32(packed: Tensor, num_bits: int, shape) -> Tensor:
+    pf = 32 // num_bits
+    w = packed.to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(pf, dtype=torch.int64) * num_bits
+    u = (w[..., None] >> shifts) & ((1 << num_bits) - 1)
+    u = u.reshape(packed.shape[0], -1)[:, : shape[1]]
+    return (u - (1 << (num_bits - 1))).to(torch.int8)
+
+
+def pack_weight(weight: dict, bits: int, sym: bool, group_size: Optional[int] = None) -> dict:
+    """pack_quantized_model.py:57-75."""
+    qweight, scale, zero = weight["qweight"], weight["scale"], weight["zero"]
+    group_size = group_size or qweight.shape[-1]
+    shifted = qweight.to(torch.int8) - zero.repeat_interleave(group_size, dim=-1).to(torch.int8)  # :66
+    out = {
+        "weight_packed": pack_to_int32(shifted, bits),  # :67
+        "weight_shape": torch.tensor(qweight.shape),  # :70
+        "weight_scale": scale,  # :71
+    }
+    if not sym:
+        out["weight_zero_point"] = weight["zero"]  # :73-74
+    return out

@@ -1,0 +1,263 @@
+"""Kernel-level parity: each C-ABI entry point against the CPU oracle on the same seeded inputs."""
+import pytest
+import torch
+
+from moe_quant_amd import ops, synth
+from oracle import gptq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def _rand(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+# ---------------------------------------------------------------- fp32 MFMA GEMM building block
+@pytest.mark.parametrize("a_kc,b_kc", [(True, True), (True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (300, 200, 72), (64, 576, 128), (513, 129, 17)])
+def test_gemm_f32_layouts(dev, a_kc, b_kc, M, N, K):
+    _say(f"gemm a_kc={a_kc} b_kc={b_kc} {M}x{N}x{K}")
+    A = _rand((M, K), 1)
+    B = _rand((K, N), 2)
+    C0 = _rand((M, N), 3)
+    Ad = (A if a_kc else A.t().contiguous()).to(dev)
+    Bd = (B.t().contiguous() if b_kc else B).to(dev)
+    Cd = C0.clone().to(dev)
+    sam, sak = (K, 1) if a_kc else (1, M)
+    sbk, sbn = (1, K) if b_kc else (N, 1)
+    ops.gemm_f32_(Ad, sam, sak, Bd, sbk, sbn, Cd, M, N, K, alpha=-0.5, beta=2.0)
+    ref = 2.0 * C0.double() - 0.5 * (A.double() @ B.double())
+    err = (Cd.cpu().double() - ref).abs().max().item()
+    assert err < 1e-4 * max(1.0, ref.abs().max().item()), err
+
+
+def test_gemm_f32_tri_and_ktrim(dev):
+    n = 384
+    A = _rand((n, 128), 4)
+    C0 = _rand((n, n), 5)
+    Cd = C0.clone().to(dev)
+    Ad = A.to(dev)
+    # upper block triangle only: C -= A A^T
+    ops.gemm_f32_(Ad, 128, 1, Ad, 1, 128, Cd, n, n, 128, alpha=-1.0, beta=1.0, tri=1)
+    ref = C0.double() - A.double() @ A.double().t()
+    out = Cd.cpu().double()
+    for bi in range(3):
+        for bj in range(3):
+            blk = (slice(bi * 128, bi * 128 + 128), slice(bj * 128, bj * 128 + 128))
+            want = ref[blk] if bi <= bj else C0.double()[blk]
+            assert (out[blk] - want).abs().max().item() < 1e-3
+    # ktrim=2: A upper triangular with garbage below the block diagonal
+    T = torch.triu(_rand((n, n), 6))
+    Tg = T.clone()
+    for bi in range(3):
+        for bj in range(bi):
+            Tg[bi * 128:(bi + 1) * 128, bj * 128:(bj + 1) * 128] = float("nan")
+    B = _rand((n, 200), 7)
+    out = torch.zeros(n, 200, device=dev)
+    ops.gemm_f32_(Tg.to(dev), n, 1, B.to(dev), 200, 1, out, n, 200, n, ktrim=2)
+    assert (out.cpu().double() - T.double() @ B.double()).abs().max().item() < 1e-3
+    # ktrim=1: A(m,k) = T[k,m]
+    out = torch.zeros(n, 200, device=dev)
+    ops.gemm_f32_(Tg.to(dev), 1, n, B.to(dev), 200, 1, out, n, 200, n, ktrim=1)
+    assert (out.cpu().double() - T.double().t() @ B.double()).abs().max().item() < 1e-3
+
+
+# ---------------------------------------------------------------- (1) Hessian SYRK
+@pytest.mark.parametrize("n,C", [(1024, 896), (4096, 256), (100, 128), (33, 384), (5000, 640)])
+def test_hessian_syrk_vs_fp64(dev, n, C):
+    _say(f"syrk n={n} C={C}")
+    X = synth.activations_outlier(n, C, seed=n + C)
+    H = torch.zeros(C, C, device=dev)
+    ops.hessian_syrk_(H, X.to(dev), 0.0, 2.0 / n)
+    H64 = O.hessian_fp64([X])
+    Hc = H.cpu().double()
+    assert ((Hc - H64).norm() / H64.norm()).item() < 1e-5  # the 1e-5 Frobenius gate
+    assert torch.equal(Hc, Hc.t())  # mirrored exactly
+
+
+def test_hessian_running_mean_matches_oracle(dev):
+    C = 512
+    X = synth.activations_swiglu(3000, C, seed=9)
+    chunks = [X[:700], X[700:701], X[701:2500], X[2500:]]
+    H = torch.zeros(C, C, device=dev)
+    Href, n = None, 0
+    for x in chunks:
+        beta, alpha = n / (n + x.shape[0]), 2.0 / (n + x.shape[0])
+        ops.hessian_syrk_(H, x.to(dev), beta, alpha)
+        Href, n = O.hessian_update(Href, n, x)
+    H64 = O.hessian_fp64(chunks)
+    assert ((H.cpu().double() - H64).norm() / H64.norm()).item() < 1e-5
+    assert ((H.cpu() - Href).norm() / Href.norm()).item() < 1e-5
+
+
+def test_hessian_upper_only(dev):
+    C, n = 256, 512
+    X = synth.activations_outlier(n, C, seed=3).to(dev)
+    H = torch.full((C, C), 7.0, device=dev)
+    ops.hessian_syrk_(H, X, 0.0, 1.0, mirror=False)
+    Hc = H.cpu()
+    ref = (X.cpu().double().t() @ X.cpu().double())
+    assert (torch.triu(Hc).double() - torch.triu(ref)).abs().max() / ref.abs().max() < 1e-5
+    assert torch.all(Hc[128:, :128] == 7.0)  # strictly-lower off-diagonal tile untouched
+
+
+# ---------------------------------------------------------------- (2) factorisation
+def _spd(C, seed, n=None):
+    X = synth.activations_outlier(n or (C + C // 8), C, seed)
+    H, _ = O.hessian_update(None, 0, X)
+    H.diagonal().add_(0.01 * H.diag().mean())
+    return H
+
+
+@pytest.mark.parametrize("C", [128, 256, 384, 896, 1024])
+def test_factor_vs_torch_chain(dev, C):
+    _say(f"factor C={C}")
+    H = _spd(C, C)
+    Hi = torch.cholesky_inverse(torch.linalg.cholesky(H.double()))
+    U64 = torch.linalg.cholesky(Hi, upper=True)
+    U64 = U64 / U64.diag()[:, None]
+    A = H.clone().to(dev)
+    info = ops.factor_upper_inverse_(A)
+    assert int(info.item()) == 0
+    U = A.cpu()
+    assert torch.equal(torch.tril(U, -1), torch.zeros_like(U))
+    assert torch.equal(U.diag(), torch.ones(C))
+    rel = ((U.double() - U64).norm() / U64.norm()).item()
+    # the fp32 torch chain itself sits at ~1e-6 from the fp64 answer
+    Hi32 = torch.cholesky_inverse(torch.linalg.cholesky(H))
+    U32 = torch.linalg.cholesky(Hi32, upper=True)
+    U32 = U32 / U32.diag()[:, None]
+    rel32 = ((U32.double() - U64).norm() / U64.norm()).item()
+    _say(f"  rel err vs fp64: ours {rel:.2e}, torch fp32 chain {rel32:.2e}")
+    assert rel < max(5e-6, 5 * rel32)
+
+
+def test_factor_reports_non_pd(dev):
+    C = 256
+    H = _spd(C, 77)
+    H[200, 200] = -1.0
+    A = H.to(dev)
+    info = ops.factor_upper_inverse_(A)
+    assert int(info.item()) == 201
+    H = _spd(C, 78)
+    H[5, 9] = float("nan")
+    info = ops.factor_upper_inverse_(H.to(dev))
+    assert int(info.item()) != 0
+
+
+def test_inv_sym(dev):
+    from moe_quant_amd.linalg_utils import inv_sym
+
+    for C in (200, 384):
+        H = _spd(C, 5 + C)
+        Hi = inv_sym(H.to(dev)).cpu().double()
+        ref = torch.linalg.inv(H.double())
+        assert ((Hi - ref).norm() / ref.norm()).item() < 1e-4
+    with pytest.raises(torch.linalg.LinAlgError):
+        inv_sym(-torch.eye(128, device=dev))
+
+
+# ---------------------------------------------------------------- (3) grid / layout / loop
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("g", [32, 128, 384])
+def test_grid_bit_exact(dev, dtype, g):
+    R, C = 96, 768
+    W = (_rand((R, C), 11, 0.02)).to(dtype)
+    W[3, 128:256] = 0  # all-zero group -> bf16(1e-12)
+    rd = torch.bfloat16 if dtype == torch.float32 else dtype
+    s_ref, z_ref, maxq = O.quantization_grid(W.float(), g, 4, rd)
+    s_rg, s_gr = ops.quant_grid_sym(W.to(dev), g, 4, rd)
+    assert torch.equal(s_rg.cpu(), s_ref)
+    assert torch.equal(s_gr.cpu(), s_ref.t())
+
+
+def test_prepare_and_untranspose(dev):
+    R, C = 200, 320
+    W = _rand((R, C), 12, 0.02).bfloat16()
+    perm = torch.randperm(C, generator=torch.Generator().manual_seed(1))
+    dead = torch.zeros(C, dtype=torch.uint8)
+    dead[[3, 77]] = 1
+    Wt = ops.prepare_wt(W.to(dev), perm.to(torch.int32).to(dev), dead.to(dev)).cpu()
+    ref = W.float().clone()
+    ref[:, dead.bool()] = 0
+    assert torch.equal(Wt, ref.t()[perm])
+    Q = torch.randint(0, 16, (C, R), dtype=torch.uint8)
+    perm_inv = torch.argsort(perm)
+    codes = ops.untranspose_codes(Q.to(dev), perm_inv.to(torch.int32).to(dev)).cpu()
+    assert torch.equal(codes, Q[perm_inv].t())
+    packed = ops.pack_from_qt(Q.to(dev), perm_inv.to(torch.int32).to(dev)).cpu()
+    assert torch.equal(packed, O.pack_to_int32(codes.to(torch.int8) - 8, 4))
+
+
+def _loop_case(R, C, seed, g=128, act_order=False):
+    W = synth.weight(R, C, seed)
+    X = synth.activations_outlier(C + C // 4, C, seed + 1)
+    H, _ = O.hessian_update(None, 0, X)
+    H, W32, _, _ = O.quantization_pre_step(H, W)
+    s, z, maxq = O.quantization_grid(W32, g, 4, torch.bfloat16)
+    s_rep, z_rep = O.replicate_grid(s, z, g)
+    perm, perm_inv = O.act_order_perm(H, act_order)
+    Hp = H[perm][:, perm]
+    U, ok = O.hessian_inverse(Hp, W32, 0.01)
+    return W32, U, s, s_rep, z_rep, maxq, perm, perm_inv
+
+
+@pytest.mark.parametrize("R,C,block", [(256, 512, 128), (100, 384, 128), (64, 300, 128), (130, 256, 64), (64, 128, 128)])
+def test_loop_vs_oracle_same_U(dev, R, C, block):
+    _say(f"loop R={R} C={C} block={block}")
+    W32, U, s, s_rep, z_rep, maxq, perm, _ = _loop_case(R, C, 31 + R)
+    Wt_ref = W32.t()[perm].contiguous()
+    q_ref = O.gptq_loop(Wt_ref, U, s_rep.t()[perm].contiguous(), z_rep.t()[perm].contiguous(), maxq,
+                        torch.bfloat16, block)
+    Wt = W32.t()[perm].contiguous().to(dev)
+    st = s_rep.t()[perm].contiguous().to(dev)
+    zt = z_rep.t()[perm].contiguous().to(dev)
+    Qt = ops.gptq_loop_(Wt, U.to(dev), st, None, zt, 0.0, 15.0, torch.bfloat16, block)
+    match = (Qt.cpu().float() == q_ref).float().mean().item()
+    _say(f"  code match {match:.6f}")
+    assert match >= 0.999
+    # dequantized weights written back must equal (q - 8) * s exactly
+    assert torch.equal(Wt.cpu(), ((Qt.cpu().float() - 8.0) * st.cpu()).bfloat16().float())
+
+
+def test_loop_identity_U_is_round_to_nearest(dev):
+    R, C = 128, 256
+    W32, _, s, s_rep, z_rep, maxq, _, _ = _loop_case(R, C, 5)
+    Wt = W32.t().contiguous().to(dev)
+    st = s_rep.t().contiguous().to(dev)
+    Qt = ops.gptq_loop_(Wt, torch.eye(C, device=dev), st, None, None, 8.0, 15.0, torch.bfloat16, 128)
+    want = torch.floor(W32.t() / s_rep.t() + 8.5).clamp(0, 15)
+    assert torch.equal(Qt.cpu().float(), want)
+
+
+def test_loop_compact_scale_and_perm(dev):
+    R, C, g = 128, 512, 64
+    W32, U, s, s_rep, z_rep, maxq, perm, perm_inv = _loop_case(R, C, 8, g=g, act_order=True)
+    Wt_ref = W32.t()[perm].contiguous()
+    q_ref = O.gptq_loop(Wt_ref, U, s_rep.t()[perm].contiguous(), z_rep.t()[perm].contiguous(), maxq,
+                        torch.bfloat16, 128)
+    Wt = ops.prepare_wt(W32.to(dev), perm.to(torch.int32).to(dev))
+    scale_row = (perm // g).to(torch.int32).to(dev)
+    Qt = ops.gptq_loop_(Wt, U.to(dev), s.t().contiguous().to(dev), scale_row, None, 8.0, 15.0, torch.bfloat16, 128)
+    assert (Qt.cpu().float() == q_ref).float().mean().item() >= 0.999
+
+
+# ---------------------------------------------------------------- (4) packer
+@pytest.mark.parametrize("R,C", [(64, 128), (7, 24), (33, 100), (5, 7), (1, 8), (256, 2048)])
+def test_pack_bit_exact(dev, R, C):
+    q = torch.randint(0, 16, (R, C), dtype=torch.uint8, generator=torch.Generator().manual_seed(R * C))
+    want = O.pack_to_int32(q.to(torch.int8) - 8, 4)
+    got = ops.pack_int4(q.to(dev)).cpu()
+    assert torch.equal(got, want)
+    # explicit zero points (the general form pack_weight uses)
+    g = C if C % 8 else 8
+    zero = torch.full((R, C // g), 8.0)
+    got = ops.pack_int4(q.to(dev), zero.to(dev), g).cpu()
+    assert torch.equal(got, want)
+    # round trip
+    assert torch.equal(O.unpack_from_int32(got, 4, (R, C)) + 8, q.to(torch.int8))
