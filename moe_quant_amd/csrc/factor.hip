@@ -25,7 +25,7 @@ constexpr int LDD = 129;
 // One workgroup, 256 threads.  Block is staged in LDS; on exit the global block holds R_bb^-1
 // (upper, zeros below the diagonal).  A non-positive or NaN pivot records its 1-based global index
 // in *info (first one wins) and is replaced by 1 so that every wave still finishes normally.
-__global__ __launch_bounds__(256) void revchol_diag_kernel(float* __restrict__ A, long ld, int i1, int* info) {
+__global__ __launch_bounds__(256) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* S = reinterpret_cast<float*>(smem);  // [NB][LDD]
   float* colj = S + NB * LDD;                 // [NB]
@@ -85,13 +85,16 @@ __global__ __launch_bounds__(256) void revchol_diag_kernel(float* __restrict__ A
 }
 
 // U[j,k] <- U[j,k] / U[j,j] for k > j, 1 on the diagonal, 0 for k < j (normalize == 0: only the zeroing).
-// One workgroup per row so the
-// diagonal is read by every thread before any thread overwrites it.
-__global__ __launch_bounds__(256) void unit_diag_kernel(float* __restrict__ A, long ld, int C, int normalize) {
+// One workgroup per row.  The diagonal travels through LDS: the one thread that loads it publishes the
+// value before the barrier (a data dependence the compiler cannot reorder), so the thread that later
+// overwrites the diagonal cannot be observed by anyone.
+__global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C, int normalize) {
+  __shared__ float dsh;
   const int j = blockIdx.x;
   float* row = A + (long)j * ld;
-  const float d = row[j];
+  if (threadIdx.x == 0) dsh = row[j];
   __syncthreads();
+  const float d = dsh;
   if (normalize) {
     for (int k = threadIdx.x; k < C; k += 256) row[k] = (k > j) ? (row[k] / d) : (k == j ? 1.f : 0.f);
   } else {

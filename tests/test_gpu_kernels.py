@@ -204,13 +204,15 @@ def _loop_case(R, C, seed, g=128, act_order=False):
     perm, perm_inv = O.act_order_perm(H, act_order)
     Hp = H[perm][:, perm]
     U, ok = O.hessian_inverse(Hp, W32, 0.01)
-    return W32, U, s, s_rep, z_rep, maxq, perm, perm_inv
+    return W32, U.contiguous(), s, s_rep, z_rep, maxq, perm, perm_inv
 
 
-@pytest.mark.parametrize("R,C,block", [(256, 512, 128), (100, 384, 128), (64, 300, 128), (130, 256, 64), (64, 128, 128)])
-def test_loop_vs_oracle_same_U(dev, R, C, block):
-    _say(f"loop R={R} C={C} block={block}")
-    W32, U, s, s_rep, z_rep, maxq, perm, _ = _loop_case(R, C, 31 + R)
+@pytest.mark.parametrize(
+    "R,C,block,g", [(256, 512, 128, 128), (100, 384, 128, 128), (64, 300, 128, 100), (130, 256, 64, 128), (64, 128, 128, 128)]
+)
+def test_loop_vs_oracle_same_U(dev, R, C, block, g):
+    _say(f"loop R={R} C={C} block={block} g={g}")
+    W32, U, s, s_rep, z_rep, maxq, perm, _ = _loop_case(R, C, 31 + R, g=g)
     Wt_ref = W32.t()[perm].contiguous()
     q_ref = O.gptq_loop(Wt_ref, U, s_rep.t()[perm].contiguous(), z_rep.t()[perm].contiguous(), maxq,
                         torch.bfloat16, block)
