@@ -20,68 +20,163 @@
 namespace {
 
 constexpr int NB = 128;
-constexpr int LDD = 129;
+constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
+constexpr int LDM = 131;   // LDS row pitch (odd: lane-per-row accesses hit 32 distinct banks)
 
-// One workgroup, 256 threads.  Block is staged in LDS; on exit the global block holds R_bb^-1
-// (upper, zeros below the diagonal).  A non-positive or NaN pivot records its 1-based global index
-// in *info (first one wins) and is replaced by 1 so that every wave still finishes normally.
-__global__ __launch_bounds__(256) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* S = reinterpret_cast<float*>(smem);  // [NB][LDD]
-  float* colj = S + NB * LDD;                 // [NB]
-  float* part = colj + NB;                    // [256]
-  const int tid = threadIdx.x;
-  float* blk = A + (long)i1 * ld + i1;
+// ---------------------------------------------------------------------------------------------
+// Diagonal block: S (128x128, upper valid) -> R^-1 where S = R R^T, R upper.
+//
+// One LDS array holds two triangular matrices side by side: the upper triangle S(i,k), k >= i, at
+// column k+1, and below it Xt(c,k) = X[k][c], k <= c, at column k, where X accumulates R^-1.
+// Stacking M = [S; Xt] makes the inverse fall out of the factorisation: every elimination step that
+// scales column j of S by 1/R_jj and subtracts its outer product from the columns to its left does,
+// applied unchanged to the rows of Xt (initialised to the identity), exactly the right-looking update
+// of the triangular inverse.  Nothing extra is computed for the inverse except more rows.
+//
+// Sub-blocks of 32: the 32x32 diagonal sub-block is eliminated by one wavefront with a row per lane in
+// registers -- lanes 0-31 carry S rows, lanes 32-63 the matching Xt rows, same instructions -- and the
+// off-diagonal work (column scaling by the sub-block inverse, outer-product updates) runs as 32x32x32
+// products on the fp32 matrix cores, one product per wavefront at a time.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float& Sv(float* buf, int i, int k) { return buf[i * LDM + k + 1]; }
+__device__ __forceinline__ float& Xv(float* buf, int c, int k) { return buf[c * LDM + k]; }
+
+__device__ __forceinline__ float bcast_lane(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+template <int J>
+struct ElimStep {
+  // one elimination step on column J of the 32x32 sub-block held one row per lane in reg[]
+  static __device__ __forceinline__ void run(float (&reg)[SB], int gidx, int* info, int lane) {
+    float d = bcast_lane(reg[J], J);
+    if (!(d > 0.f)) {
+      if (lane == 0) atomicCAS(info, 0, gidx + J + 1);
+      d = 1.f;
+    }
+    float y = __frsqrt_rn(d);
+    y = y * (1.5f - 0.5f * d * y * y);  // one Newton step: 1/sqrt(d) to fp32 accuracy
+    const float v = reg[J] * y;
+    reg[J] = v;
+#pragma unroll
+    for (int k = 0; k < J; ++k) reg[k] = fmaf(-bcast_lane(v, k), v, reg[k]);
+    ElimStep<J - 1>::run(reg, gidx, info, lane);
+  }
+};
+template <>
+struct ElimStep<-1> {
+  static __device__ __forceinline__ void run(float (&)[SB], int, int*, int) {}
+};
+
+// acc (32x32, MFMA layout) (+)= sum_k a(m,k) * b(k,n); a/b fetch one element for this lane
+template <typename FA, typename FB>
+__device__ __forceinline__ void mm32(floatx16& acc, FA a, FB b, int lane) {
+  const int x = lane & 31, kk = lane >> 5;
+  float av[16], bv[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    av[t] = a(x, 2 * t + kk);
+    bv[t] = b(2 * t + kk, x);
+  }
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], bv[t], acc, 0, 0, 0);
+}
+
+// buf: LDS, NB*LDM floats.  blk: global 128x128 block (row pitch ld).  gidx0: global index of its first row.
+__device__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int idx = tid; idx < NB * NB; idx += 256) {
     const int r = idx >> 7, c = idx & 127;
-    S[r * LDD + c] = (c >= r) ? blk[(long)r * ld + c] : 0.f;
+    if (c >= r) Sv(buf, r, c) = blk[(long)r * ld + c];
+    else Xv(buf, r, c) = 0.f;  // strictly lower part of Xt starts at zero (the unit diagonal is implicit)
   }
   __syncthreads();
 
-  const int k = tid & 127, h = tid >> 7;
-  // ---- reverse Cholesky: S = R R^T, R upper, columns from last to first
-  for (int j = NB - 1; j >= 0; --j) {
-    float d = S[j * LDD + j];
-    if (!(d > 0.f)) {
-      if (tid == 0) atomicCAS(info, 0, i1 + j + 1);
-      d = 1.f;
-    }
-    const float r = sqrtf(d);
-    float ck = 0.f;
-    if (h == 0) {
-      if (k < j) ck = S[k * LDD + j] / r;
-      else if (k == j) ck = r;
-      colj[k] = ck;
+  for (int J = NB / SB - 1; J >= 0; --J) {
+    const int o = J * SB;
+    if (wave == 0) {
+      float reg[SB];
+      const int li = lane & 31;
+      const bool up = lane >= 32;
+#pragma unroll
+      for (int k = 0; k < SB; ++k) reg[k] = up ? (k == li ? 1.f : 0.f) : (k >= li ? Sv(buf, o + li, o + k) : 0.f);
+      ElimStep<SB - 1>::run(reg, gidx0 + o, info, lane);
+#pragma unroll
+      for (int k = 0; k < SB; ++k) {
+        if (!up && k >= li) Sv(buf, o + li, o + k) = reg[k];
+        if (up && k <= li) Xv(buf, o + li, o + k) = reg[k];
+      }
     }
     __syncthreads();
-    if (h == 0 && k <= j) S[k * LDD + j] = ck;
-    ck = colj[k];
-    if (k < j) {
-      for (int i = h; i <= k; i += 2) S[i * LDD + k] = fmaf(-colj[i], ck, S[i * LDD + k]);
+    // ---- column block J of M times the sub-block inverse: V = M(:,J) * Xinv^T, Xinv[n][k] = Xt(o+k... ) masked
+    {
+      const int ntask = 3;  // J row blocks of S above the diagonal + (3-J) row blocks of Xt below it
+      for (int t = wave; t < ntask; t += 4) {
+        const bool is_s = t < J;
+        const int rb = is_s ? t : (t + 1);  // S row block I=t, or Xt row block Cb=t+1 (> J)
+        const int ro = rb * SB;
+        floatx16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        auto bfn = [&](int k, int n) { return (k >= n) ? Xv(buf, o + k, o + n) : 0.f; };  // Xinv[n][k]
+        if (is_s) mm32(acc, [&](int m, int k) { return Sv(buf, ro + m, o + k); }, bfn, lane);
+        else mm32(acc, [&](int m, int k) { return Xv(buf, ro + m, o + k); }, bfn, lane);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
+          if (is_s) Sv(buf, ro + m, o + n) = acc[v];
+          else Xv(buf, ro + m, o + n) = acc[v];
+        }
+      }
+    }
+    __syncthreads();
+    // ---- outer-product updates of the column blocks K < J:  M(rb,K) -= V(rb) * R(K,J)^T
+    {
+      // tasks enumerated as (K, rb): for each K < J the S row blocks I <= K, then the Xt row blocks Cb >= J
+      const int per_k_x = NB / SB - J;
+      int t = 0;
+      for (int K = 0; K < J; ++K) {
+        const int cnt = (K + 1) + per_k_x;
+        for (int q = 0; q < cnt; ++q, ++t) {
+          if ((t & 3) != wave) continue;
+          const bool is_s = q <= K;
+          const int rb = is_s ? q : (J + (q - K - 1));
+          const int ro = rb * SB, ko = K * SB;
+          floatx16 acc;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
+            acc[v] = is_s ? Sv(buf, ro + m, ko + n) : Xv(buf, ro + m, ko + n);
+          }
+          auto bfn = [&](int k, int n) { return Sv(buf, ko + n, o + k); };  // R(K,J)[n][k]
+          if (is_s) {
+            mm32(acc, [&](int m, int k) { return -Sv(buf, ro + m, o + k); }, bfn, lane);
+          } else if (rb == J) {  // V is the sub-block inverse itself; only its lower triangle is Xt data
+            mm32(acc, [&](int m, int k) { return (k <= m) ? -Xv(buf, ro + m, o + k) : 0.f; }, bfn, lane);
+          } else {
+            mm32(acc, [&](int m, int k) { return -Xv(buf, ro + m, o + k); }, bfn, lane);
+          }
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
+            if (is_s) Sv(buf, ro + m, ko + n) = acc[v];
+            else Xv(buf, ro + m, ko + n) = acc[v];
+          }
+        }
+      }
     }
     __syncthreads();
   }
-  // ---- in-place inverse of the upper-triangular R, column by column:
-  //      X[i,j] = -(sum_{k=i}^{j-1} X[i,k] R[k,j]) / R[j,j],  X[j,j] = 1/R[j,j]
-  for (int j = 0; j < NB; ++j) {
-    const int i = k;
-    float s = 0.f;
-    if (i < j) {
-      for (int kk = i + h; kk < j; kk += 2) s = fmaf(S[i * LDD + kk], S[kk * LDD + j], s);
-    }
-    part[tid] = s;
-    const float rjj = S[j * LDD + j];
-    __syncthreads();
-    if (h == 0) {
-      if (i < j) S[i * LDD + j] = -(part[i] + part[i + 128]) / rjj;
-      else if (i == j) S[j * LDD + j] = 1.f / rjj;
-    }
-    __syncthreads();
-  }
+  // R^-1[r][c] = Xt(c, r) for r <= c, zero below the diagonal
   for (int idx = tid; idx < NB * NB; idx += 256) {
     const int r = idx >> 7, c = idx & 127;
-    blk[(long)r * ld + c] = S[r * LDD + c];
+    blk[(long)r * ld + c] = (r <= c) ? Xv(buf, c, r) : 0.f;
   }
+}
+
+__global__ __launch_bounds__(256) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info);
 }
 
 // U[j,k] <- U[j,k] / U[j,j] for k > j, 1 on the diagonal, 0 for k < j (normalize == 0: only the zeroing).
@@ -102,7 +197,7 @@ __global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C
   }
 }
 
-constexpr size_t DIAG_SMEM = (size_t)(NB * LDD + NB + 256) * sizeof(float);
+constexpr size_t DIAG_SMEM = (size_t)(NB * LDM) * sizeof(float);
 
 }  // namespace
 
