@@ -21,11 +21,11 @@ namespace {
 
 constexpr int B = 128;
 
-template <int RD>
-__device__ __forceinline__ float round_dtype(float x) {
-  if (RD == 1) return round_to_bf16(x);
-  if (RD == 2) return __half2float(__float2half_rn(x));
-  return x;
+__device__ __forceinline__ float round_dtype(float x, int rd) {
+  // branch-free so that the unrolled column steps stay one basic block
+  const float b = round_to_bf16(x);
+  const float h = __half2float(__float2half_rn(x));
+  return rd == 1 ? b : (rd == 2 ? h : x);
 }
 
 struct LoopArgs {
@@ -39,77 +39,150 @@ struct LoopArgs {
   const int* scale_row;  // nullable: scale row of column j is scale_row[j], else j
   const float* qzero;    // nullable: same indexing as scale, else qzero_const
   float qzero_const, maxq;
+  int rd;
   uint8_t* Qt;
   float* E;
 };
 
-constexpr int MB = 16;      // micro-block: columns walked with weights in registers
-constexpr int WSTRIDE = 64; // LDS tile is [column][lane]
+constexpr int MB = 16;       // micro-block: columns walked with weights in registers
+constexpr int WSTRIDE = 64;  // weight tile in LDS is [column][lane]
+constexpr int UL = 132;      // pitch of the U block in LDS (16-byte aligned rows)
 
-typedef const float __attribute__((address_space(4))) * cfloat_p;  // constant address space -> scalar loads
+typedef const int __attribute__((address_space(4))) * cint_p;  // constant address space: scalar loads
 
 // One wavefront owns 64 rows.  The 128-column block of those rows sits in LDS ([column][lane], so
-// every access is conflict-free); 16 columns at a time move to registers for the strictly sequential
-// part, and their 16 errors are then folded into the rest of the block, 16 columns per pass, with the
-// multipliers U[j,k] arriving as scalar operands.  For every weight the updates are applied in
-// ascending j with one fma each, exactly the order of the sequential reference.
-template <bool FULL, int RD>
-__global__ __launch_bounds__(64) void gptq_block_kernel(LoopArgs a, int i1, int nb) {
-  __shared__ float tile[B * WSTRIDE];
+// every access is conflict-free) next to the 128x128 block of U.  16 columns at a time move to
+// registers for the strictly sequential part; their 16 errors are then folded into the rest of the
+// block, 16 columns per pass.  The multipliers U[j,k] are the same for every lane: they are read from
+// LDS with all lanes on one address (a broadcast, four values per read).  For every weight the updates
+// are applied in ascending j with one fma each, exactly the order of the sequential reference.
+//
+// A lone wavefront per CU cannot hide latency by switching waves, so every phase issues its loads in
+// bulk before the first use: the kernel is built from branch-free unrolled blocks for that reason
+// (ROWMAP / QZERO are template flags, the rounding mode is a select).
+template <bool FULL, bool ROWMAP, bool QZERO>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void gptq_block_kernel(LoopArgs a, int i1,
+                                                                                                  int nb) {
+  __shared__ __attribute__((aligned(16))) float tile[B * WSTRIDE];
+  __shared__ __attribute__((aligned(16))) float ut[B * UL];
   const int lane = threadIdx.x;
   const int r0 = blockIdx.x * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
-  // does, which keeps every branch wave-uniform (a divergent branch would turn the scalar loads of U
-  // into per-lane vector loads).
+  // does, so no branch in this kernel ever diverges.
   const int r = min(r0 + lane, a.R - 1);
   float* __restrict__ wp = a.Wt + (long)i1 * a.ldw + r;
-  for (int k = 0; k < B; ++k) tile[k * WSTRIDE + lane] = (FULL || k < nb) ? wp[(long)k * a.ldw] : 0.f;
-  cfloat_p U = (cfloat_p)(a.U);
-  const float maxq = a.maxq;
-#pragma unroll 1
-  for (int c0 = 0; c0 < (FULL ? B : nb); c0 += MB) {
-    float w[MB], e[MB];
 #pragma unroll
-    for (int t = 0; t < MB; ++t) w[t] = tile[(c0 + t) * WSTRIDE + lane];
+  for (int kb = 0; kb < B; kb += 32) {
+    float t[32];
 #pragma unroll
-    for (int J = 0; J < MB; ++J) {
-      e[J] = 0.f;
-      if (FULL || c0 + J < nb) {
-        const int col = i1 + c0 + J;
-        const int srow = a.scale_row ? a.scale_row[col] : col;
-        const float s = a.scale[(long)srow * a.lds + r];
-        const float z = a.qzero ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
-        const float x = w[J];
-        const float v = x / s + z;
-        float q = floorf(v + 0.5f);
-        q = fminf(fmaxf(q, 0.f), maxq);
-        const float y = round_dtype<RD>((q - z) * s);
-        e[J] = y - x;
-        wp[(long)(c0 + J) * a.ldw] = y;
-        a.Qt[(long)col * a.R + r] = (uint8_t)q;
-        a.E[(long)(c0 + J) * a.R + r] = e[J];
-        cfloat_p urow = U + (long)col * a.ldu + i1 + c0;
+    for (int k = 0; k < 32; ++k) t[k] = (FULL || kb + k < nb) ? wp[(long)(kb + k) * a.ldw] : 0.f;
 #pragma unroll
-        for (int t = J + 1; t < MB; ++t) {
-          const int tc = FULL ? t : min(t, nb - 1 - c0);  // keep the scalar load inside the matrix
-          w[t] = fmaf(urow[tc], e[J], w[t]);
+    for (int k = 0; k < 32; ++k) tile[(kb + k) * WSTRIDE + lane] = t[k];
+  }
+  {
+    const float* __restrict__ Ub = a.U + (long)i1 * a.ldu + i1;
+    const bool vec = FULL && ((a.ldu & 3) == 0) && ((((uintptr_t)Ub) & 15) == 0);
+    if (vec) {
+#pragma unroll
+      for (int it = 0; it < B * (B / 4) / 64; it += 16) {
+        float4 v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = lane + (it + u) * 64;
+          const int j = idx >> 5, k = (idx & 31) << 2;
+          v[u] = (k + 3 > j) ? *reinterpret_cast<const float4*>(Ub + (long)j * a.ldu + k) : make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          const int idx = lane + (it + u) * 64;
+          const int j = idx >> 5, k = (idx & 31) << 2;
+          *reinterpret_cast<float4*>(&ut[j * UL + k]) = v[u];
         }
       }
+    } else {
+      for (int idx = lane; idx < B * B; idx += 64) {
+        const int j = idx >> 7, k = idx & 127;
+        ut[j * UL + k] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
+      }
     }
-    const int cend = FULL ? B : nb;
+  }
+  __syncthreads();
+  const float maxq = a.maxq;
+  const int rd = a.rd;
+  const int cend = FULL ? B : nb;
+  cint_p srp = (cint_p)(a.scale_row);
+#pragma unroll 1
+  for (int c0 = 0; c0 < cend; c0 += MB) {
+    float w[MB], e[MB], sc[MB], zz[MB];
+    float4 um[MB][MB / 4];
+#pragma unroll
+    for (int t = 0; t < MB; ++t) {
+      const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
+      const int srow = ROWMAP ? srp[col] : col;
+      sc[t] = a.scale[(long)srow * a.lds + r];
+      zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
+      w[t] = tile[(c0 + t) * WSTRIDE + lane];
+    }
+#pragma unroll
+    for (int J = 0; J < MB; ++J)
+#pragma unroll
+      for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
+        um[J][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + J) * UL + c0 + 4 * t4]);
+#pragma unroll
+    for (int J = 0; J < MB; ++J) {
+      const float s = sc[J], z = zz[J];
+      const float x = w[J];
+      const float v = x / s + z;
+      float q = floorf(v + 0.5f);
+      q = fminf(fmaxf(q, 0.f), maxq);
+      const float y = round_dtype((q - z) * s, rd);
+      e[J] = (FULL || c0 + J < nb) ? (y - x) : 0.f;
+      if (FULL || c0 + J < nb) {
+        wp[(long)(c0 + J) * a.ldw] = y;
+        a.Qt[(long)(i1 + c0 + J) * a.R + r] = (uint8_t)q;
+        a.E[(long)(c0 + J) * a.R + r] = e[J];
+      }
+#pragma unroll
+      for (int t = J + 1; t < MB; ++t) {
+        const float4 u4 = um[J][t >> 2];
+        const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
+        w[t] = fmaf(u, e[J], w[t]);
+      }
+    }
+    // fold the 16 errors into the remaining columns of the block, 16 columns per pass; U rows are
+    // fetched four at a time, one group ahead of the FMAs that consume them
 #pragma unroll 1
     for (int k0 = c0 + MB; k0 < cend; k0 += MB) {
       float x[MB];
+      float4 ug[2][4][MB / 4];
 #pragma unroll
       for (int t = 0; t < MB; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
 #pragma unroll
-      for (int J = 0; J < MB; ++J) {
-        const int jr = FULL ? J : min(J, nb - 1 - c0);  // rows past the block carry e = 0; stay inside U
-        cfloat_p urow = U + (long)(i1 + c0 + jr) * a.ldu + i1 + k0;
+      for (int jj = 0; jj < 4; ++jj)
 #pragma unroll
-        for (int t = 0; t < MB; ++t) {
-          const int tc = FULL ? t : min(t, nb - 1 - k0);
-          x[t] = fmaf(urow[tc], e[J], x[t]);
+        for (int t4 = 0; t4 < MB / 4; ++t4)
+          ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + jj) * UL + k0 + 4 * t4]);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g < 3) {
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int t4 = 0; t4 < MB / 4; ++t4)
+              ug[(g + 1) & 1][jj][t4] =
+                  *reinterpret_cast<const float4*>(&ut[(c0 + 4 * (g + 1) + jj) * UL + k0 + 4 * t4]);
+        }
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const float ej = e[4 * g + jj];
+#pragma unroll
+          for (int t4 = 0; t4 < MB / 4; ++t4) {
+            const float4 u = ug[g & 1][jj][t4];
+            x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
+            x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
+            x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
+            x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
+          }
         }
       }
 #pragma unroll
@@ -118,16 +191,16 @@ __global__ __launch_bounds__(64) void gptq_block_kernel(LoopArgs a, int i1, int 
   }
 }
 
-template <int RD>
+template <bool ROWMAP, bool QZERO>
 int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   const int grid = (a.R + 63) / 64;
   for (int i1 = 0; i1 < a.C; i1 += block) {
     const int i2 = (i1 + block < a.C) ? i1 + block : a.C;
     const int nb = i2 - i1;
     if (nb == B)
-      hipLaunchKernelGGL((gptq_block_kernel<true, RD>), dim3(grid), dim3(64), 0, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid), dim3(64), 0, st, a, i1, nb);
     else
-      hipLaunchKernelGGL((gptq_block_kernel<false, RD>), dim3(grid), dim3(64), 0, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid), dim3(64), 0, st, a, i1, nb);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     if (i2 < a.C) {
@@ -149,11 +222,8 @@ extern "C" int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, l
   if (ldw < R || ldu < C || ld_scale < R) return MQ_ERR_ARG;
   if (round_dtype < 0 || round_dtype > 2) return MQ_ERR_ARG;
   if (block <= 0 || block > B) block = B;  // wider blocks only reassociate the trailing sums
-  LoopArgs a{Wt, ldw, C, R, U, ldu, scale, ld_scale, scale_row, qzero, qzero_const, maxq, Qt, E};
+  LoopArgs a{Wt, ldw, C, R, U, ldu, scale, ld_scale, scale_row, qzero, qzero_const, maxq, round_dtype, Qt, E};
   hipStream_t st = (hipStream_t)stream;
-  switch (round_dtype) {
-    case 0: return run_loop<0>(a, block, st);
-    case 1: return run_loop<1>(a, block, st);
-    default: return run_loop<2>(a, block, st);
-  }
+  if (scale_row) return qzero ? run_loop<true, true>(a, block, st) : run_loop<true, false>(a, block, st);
+  return qzero ? run_loop<false, true>(a, block, st) : run_loop<false, false>(a, block, st);
 }
