@@ -51,3 +51,4 @@ struct GemmF32 {
   long batchA, batchB, batchC;
 };
 int mq_launch_gemm_f32(const GemmF32& g, hipStream_t stream);
+bool mq_gemm_operand_aligned(const float* p, long ld, long batch);
