@@ -15,7 +15,7 @@
 //     T^T = U22^T R12^T  (written to the unused mirror position below the diagonal)
 //     U12 = -U11 T
 //   finalize: U[j, k] /= U[j, j], strictly lower part zeroed.
-#include "common.hpp"
+#include "gemm_f32_tile.hpp"
 
 namespace {
 
@@ -48,24 +48,23 @@ __device__ __forceinline__ float bcast_lane(float v, int lane) {
 template <int J>
 struct ElimStep {
   // one elimination step on column J of the 32x32 sub-block held one row per lane in reg[]
-  static __device__ __forceinline__ void run(float (&reg)[SB], int gidx, int* info, int lane) {
+  static __device__ __forceinline__ void run(float (&reg)[SB], int gidx, int& bad) {
     float d = bcast_lane(reg[J], J);
-    if (!(d > 0.f)) {
-      if (lane == 0) atomicCAS(info, 0, gidx + J + 1);
-      d = 1.f;
-    }
+    const bool neg = !(d > 0.f);  // also catches NaN; selects, not branches: one basic block per sub-block
+    bad = (neg && bad == 0) ? (gidx + J + 1) : bad;
+    d = neg ? 1.f : d;
     float y = __frsqrt_rn(d);
     y = y * (1.5f - 0.5f * d * y * y);  // one Newton step: 1/sqrt(d) to fp32 accuracy
     const float v = reg[J] * y;
     reg[J] = v;
 #pragma unroll
     for (int k = 0; k < J; ++k) reg[k] = fmaf(-bcast_lane(v, k), v, reg[k]);
-    ElimStep<J - 1>::run(reg, gidx, info, lane);
+    ElimStep<J - 1>::run(reg, gidx, bad);
   }
 };
 template <>
 struct ElimStep<-1> {
-  static __device__ __forceinline__ void run(float (&)[SB], int, int*, int) {}
+  static __device__ __forceinline__ void run(float (&)[SB], int, int&) {}
 };
 
 // acc (32x32, MFMA layout) (+)= sum_k a(m,k) * b(k,n); a/b fetch one element for this lane
@@ -83,14 +82,30 @@ __device__ __forceinline__ void mm32(floatx16& acc, FA a, FB b, int lane) {
 }
 
 // buf: LDS, NB*LDM floats.  blk: global 128x128 block (row pitch ld).  gidx0: global index of its first row.
-__device__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info) {
+// preloaded: the caller already filled Sv (upper) and zeroed Xv (strictly lower) and synchronised.
+// blk rows must be 16-byte aligned (ld % 4 == 0).
+__device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info,
+                                                  bool preloaded) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int idx = tid; idx < NB * NB; idx += 256) {
-    const int r = idx >> 7, c = idx & 127;
-    if (c >= r) Sv(buf, r, c) = blk[(long)r * ld + c];
-    else Xv(buf, r, c) = 0.f;  // strictly lower part of Xt starts at zero (the unit diagonal is implicit)
+  if (!preloaded) {
+    float4 v[16];
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+      v[it] = *reinterpret_cast<const float4*>(blk + (long)r * ld + c);
+    }
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+      const float e[4] = {v[it].x, v[it].y, v[it].z, v[it].w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (c + q >= r) Sv(buf, r, c + q) = e[q];
+        else Xv(buf, r, c + q) = 0.f;  // strictly lower part of Xt starts at zero (unit diagonal implicit)
+      }
+    }
+    __syncthreads();
   }
-  __syncthreads();
 
   for (int J = NB / SB - 1; J >= 0; --J) {
     const int o = J * SB;
@@ -100,7 +115,9 @@ __device__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, in
       const bool up = lane >= 32;
 #pragma unroll
       for (int k = 0; k < SB; ++k) reg[k] = up ? (k == li ? 1.f : 0.f) : (k >= li ? Sv(buf, o + li, o + k) : 0.f);
-      ElimStep<SB - 1>::run(reg, gidx0 + o, info, lane);
+      int bad = 0;
+      ElimStep<SB - 1>::run(reg, gidx0 + o, bad);
+      if (bad != 0 && lane == 0) atomicCAS(info, 0, bad);
 #pragma unroll
       for (int k = 0; k < SB; ++k) {
         if (!up && k >= li) Sv(buf, o + li, o + k) = reg[k];
@@ -168,16 +185,51 @@ __device__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, in
     __syncthreads();
   }
   // R^-1[r][c] = Xt(c, r) for r <= c, zero below the diagonal
-  for (int idx = tid; idx < NB * NB; idx += 256) {
-    const int r = idx >> 7, c = idx & 127;
-    blk[(long)r * ld + c] = (r <= c) ? Xv(buf, c, r) : 0.f;
+#pragma unroll 4
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+    float4 o4;
+    o4.x = (r <= c + 0) ? Xv(buf, c + 0, r) : 0.f;
+    o4.y = (r <= c + 1) ? Xv(buf, c + 1, r) : 0.f;
+    o4.z = (r <= c + 2) ? Xv(buf, c + 2, r) : 0.f;
+    o4.w = (r <= c + 3) ? Xv(buf, c + 3, r) : 0.f;
+    *reinterpret_cast<float4*>(blk + (long)r * ld + c) = o4;
   }
 }
 
-__global__ __launch_bounds__(256) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info);
+  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false);
 }
+
+// One launch per elimination step b (block at offset i1, panel P = A[0:i1, i1:i1+128] already solved):
+//   workgroup 0        : updates the next diagonal tile (rows/cols [i1-128, i1)) with the panel, keeps the
+//                        result in LDS and inverts it right away (the next step's critical path);
+//   workgroups 1..T-1  : the other T-1 upper tiles of the trailing update  A[0:i1,0:i1] -= P P^T.
+// The diagonal-block work is thereby hidden behind the bulk of the trailing update.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void trail_diag_kernel(GemmF32 g, int total, float* A,
+                                                                                                  long ld, int i1, int* info) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* buf = reinterpret_cast<float*>(smem);
+  using namespace gemmf32;
+  if (blockIdx.x == 0) {
+    const int t = i1 / NB - 1;  // last tile of the column-major upper-triangle order
+    tile_body<true, true, true>(g, t, t, 0, buf, 1, 1, [&](int r, int c, float v) {
+      if (c >= r) Sv(buf, r, c) = v;
+    });
+    for (int idx = threadIdx.x; idx < NB * NB; idx += 256) {
+      const int r = idx >> 7, c = idx & 127;
+      if (c < r) Xv(buf, r, c) = 0.f;
+    }
+    __syncthreads();
+    diag_block_invert(buf, A + (long)(i1 - NB) * ld + (i1 - NB), ld, i1 - NB, info, true);
+  } else {
+    int tm, tn;
+    tri_decode(xcd_remap(blockIdx.x - 1, total - 1), tm, tn);
+    tile_body<true, true>(g, tm, tn, 0, buf, 1, 1);
+  }
+}
+
 
 // U[j,k] <- U[j,k] / U[j,j] for k > j, 1 on the diagonal, 0 for k < j (normalize == 0: only the zeroing).
 // One workgroup per row.  The diagonal travels through LDS: the one thread that loads it publishes the
@@ -198,6 +250,7 @@ __global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C
 }
 
 constexpr size_t DIAG_SMEM = (size_t)(NB * LDM) * sizeof(float);
+constexpr size_t FUSED_SMEM = DIAG_SMEM > gemmf32::SMEM_BYTES ? DIAG_SMEM : gemmf32::SMEM_BYTES;
 
 }  // namespace
 
@@ -209,19 +262,23 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
   if (!attr_done) {
     (void)hipFuncSetAttribute((const void*)revchol_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)DIAG_SMEM);
+    (void)hipFuncSetAttribute((const void*)trail_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)FUSED_SMEM);
     attr_done = true;
   }
+  if ((ld & 3) || ((uintptr_t)A & 15)) return MQ_ERR_ARG;  // float4 access to rows of A
   int rc;
-  for (int i1 = C - NB; i1 >= 0; i1 -= NB) {
-    hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, A, ld, i1, info);
-    if ((rc = mq_check_launch()) != MQ_OK) return rc;
-    if (i1 == 0) break;
-    float* P = A + i1;                       // panel: rows [0,i1), cols [i1, i1+NB)
+  hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, A, ld, C - NB, info);
+  if ((rc = mq_check_launch()) != MQ_OK) return rc;
+  for (int i1 = C - NB; i1 > 0; i1 -= NB) {
+    float* P = A + i1;  // panel: rows [0,i1), cols [i1, i1+NB)
     const float* Dinv = A + (long)i1 * ld + i1;
     GemmF32 panel{P, Dinv, P, ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
     if ((rc = mq_launch_gemm_f32(panel, st)) != MQ_OK) return rc;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
-    if ((rc = mq_launch_gemm_f32(trail, st)) != MQ_OK) return rc;
+    const int tiles = i1 / NB, total = tiles * (tiles + 1) / 2;
+    hipLaunchKernelGGL(trail_diag_kernel, dim3(total), dim3(256), FUSED_SMEM, st, trail, total, A, ld, i1, info);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
   for (long s = NB; s < C; s *= 2) {
     const int nfull = (int)(C / (2 * s));

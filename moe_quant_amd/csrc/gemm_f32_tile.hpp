@@ -95,8 +95,14 @@ struct TileLoader {
 // One 128x128 output tile (tm, tn) of problem g (batch index z).  smem: SMEM_BYTES of LDS.
 // The old C tile is fetched before the K loop (when beta != 0) so its latency hides behind the products;
 // it is added after the accumulation, never fed through the accumulator.
-template <bool A_KC, bool B_KC>
-__device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int z, float* smem, int vecA, int vecB) {
+// With LDS_OUT the result tile is not written to memory: it is handed to `sink(r, c, value)` (tile-local
+// coordinates) after the last LDS operand read, so the sink may overwrite the staging buffers.
+struct NoSink {
+  __device__ __forceinline__ void operator()(int, int, float) const {}
+};
+template <bool A_KC, bool B_KC, bool LDS_OUT = false, typename Sink = NoSink>
+__device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int z, float* smem, int vecA, int vecB,
+                                          Sink sink = Sink()) {
   float* As = smem;
   float* Bs = smem + 2 * STAGE;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -183,7 +189,8 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
         if (row < g.M && col < g.N) {
           float r = alpha * acc[i][j][v];
           if (beta != 0.f) r = fmaf(beta, cold[i][j][v], r);
-          C[(long)row * g.ldc + col] = r;
+          if (LDS_OUT) sink(row - m0, col - n0, r);
+          else C[(long)row * g.ldc + col] = r;
         }
       }
     }
