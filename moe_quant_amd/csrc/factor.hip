@@ -57,8 +57,10 @@ struct ElimStep {
     y = y * (1.5f - 0.5f * d * y * y);  // one Newton step: 1/sqrt(d) to fp32 accuracy
     const float v = reg[J] * y;
     reg[J] = v;
+    // nearest column first: the next step's pivot lives in reg[J-1], so its chain can start while the
+    // remaining updates of this step are still issuing
 #pragma unroll
-    for (int k = 0; k < J; ++k) reg[k] = fmaf(-bcast_lane(v, k), v, reg[k]);
+    for (int k = J - 1; k >= 0; --k) reg[k] = fmaf(-bcast_lane(v, k), v, reg[k]);
     ElimStep<J - 1>::run(reg, gidx, bad);
   }
 };

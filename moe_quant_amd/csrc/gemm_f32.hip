@@ -9,16 +9,23 @@ namespace {
 
 using namespace gemmf32;
 
+// pair_rows > 0 (triangular-K problems): the workgroup computes row tile tm and then its mirror
+// pair_rows-1-tm, so every workgroup sees the same total K and the triangle no longer unbalances the grid.
 template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int tiles_n, int total, int vecA, int vecB) {
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int tiles_n, int total, int vecA, int vecB,
+                                                      int pair_rows) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   int tm, tn;
   decode_tile(g, xcd_remap(blockIdx.x, total), tiles_n, tm, tn);
   tile_body<A_KC, B_KC>(g, tm, tn, blockIdx.z, reinterpret_cast<float*>(smem_raw), vecA, vecB);
+  if (pair_rows > 0) {
+    const int tm2 = pair_rows - 1 - tm;
+    if (tm2 != tm) tile_body<A_KC, B_KC>(g, tm2, tn, blockIdx.z, reinterpret_cast<float*>(smem_raw), vecA, vecB);
+  }
 }
 
 template <bool A_KC, bool B_KC>
-int launch(const GemmF32& g, int tiles_n, int total, int vecA, int vecB, hipStream_t stream) {
+int launch(const GemmF32& g, int tiles_n, int total, int vecA, int vecB, int pair_rows, hipStream_t stream) {
   static bool attr_done = false;
   if (!attr_done) {
     (void)hipFuncSetAttribute((const void*)gemm_f32_kernel<A_KC, B_KC>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -26,7 +33,7 @@ int launch(const GemmF32& g, int tiles_n, int total, int vecA, int vecB, hipStre
     attr_done = true;
   }
   hipLaunchKernelGGL((gemm_f32_kernel<A_KC, B_KC>), dim3(total, 1, g.batch), dim3(256), SMEM_BYTES, stream, g, tiles_n,
-                     total, vecA, vecB);
+                     total, vecA, vecB, pair_rows);
   return mq_check_launch();
 }
 
@@ -44,13 +51,18 @@ int mq_launch_gemm_f32(const GemmF32& g, hipStream_t stream) {
   if (!b_kc && g.sbn != 1) return MQ_ERR_ARG;
   if (g.tri && g.M != g.N) return MQ_ERR_ARG;
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-  const int total = g.tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  int total = g.tri ? tiles_m * (tiles_m + 1) / 2 : tiles_m * tiles_n;
+  int pair_rows = 0;
+  if (!g.tri && g.ktrim != 0 && tiles_m >= 2) {
+    pair_rows = tiles_m;
+    total = ((tiles_m + 1) / 2) * tiles_n;
+  }
   const int vecA = mq_gemm_operand_aligned(g.A, a_kc ? g.sam : g.sak, g.batchA);
   const int vecB = mq_gemm_operand_aligned(g.B, b_kc ? g.sbn : g.sbk, g.batchB);
-  if (a_kc && b_kc) return launch<true, true>(g, tiles_n, total, vecA, vecB, stream);
-  if (a_kc && !b_kc) return launch<true, false>(g, tiles_n, total, vecA, vecB, stream);
-  if (!a_kc && b_kc) return launch<false, true>(g, tiles_n, total, vecA, vecB, stream);
-  return launch<false, false>(g, tiles_n, total, vecA, vecB, stream);
+  if (a_kc && b_kc) return launch<true, true>(g, tiles_n, total, vecA, vecB, pair_rows, stream);
+  if (a_kc && !b_kc) return launch<true, false>(g, tiles_n, total, vecA, vecB, pair_rows, stream);
+  if (!a_kc && b_kc) return launch<false, true>(g, tiles_n, total, vecA, vecB, pair_rows, stream);
+  return launch<false, false>(g, tiles_n, total, vecA, vecB, pair_rows, stream);
 }
 
 // Test hook: plain GEMM through the C ABI so the MFMA core can be checked on its own.
