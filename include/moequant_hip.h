@@ -43,6 +43,10 @@ size_t mq_hessian_syrk_workspace_bytes(int n, int C);
 int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
                          int mirror, void* workspace, size_t workspace_bytes, void* stream);
 
+/* lower triangle <- transpose of the upper triangle (what mirror != 0 does after the accumulation; exported so
+ * that a caller accumulating many batches can mirror once at the end). */
+int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
+
 /* ---- (2) damped Cholesky / Cholesky-inverse -------------------------------------------------------
  * In place: A (SPD, upper triangle read, C % 128 == 0) -> unit-diagonal upper-triangular
  * U = chol(A^-1, upper) / diag, strictly lower part zeroed.  Replaces

@@ -11,6 +11,8 @@
 // partial tiles go to a caller-provided workspace and are reduced in a fixed order (deterministic).
 #include "common.hpp"
 
+extern "C" int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
+
 namespace {
 
 constexpr int T = 128;         // tile edge (channels)
@@ -192,6 +194,288 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(float* __restrict__ H,
   write_tile(H, ldh, C, tm * T, tn * T, epi, alpha, beta, mirror && tm != tn, tid);
 }
 
+// =============================================================================================
+// Large-tile kernel: 256x256 channels per workgroup, four wavefronts of 128x128 (4x4 MFMA blocks,
+// 256 accumulator registers each).  With 64x64 per wave every MFMA needs 0.5 LDS fragment reads;
+// 128x128 per wave needs 0.25, which leaves the LDS port room for the staging writes.
+//
+// Staging: 64 tokens per stage.  Each thread owns two 8-channel x 8-token patches per stage: eight
+// 16-byte loads each (32 lanes side by side read 512 contiguous bytes of one token row), an 8x8
+// transpose in registers (32 byte permutes) and eight 16-byte LDS writes, one per channel.
+// LDS layout per operand: [token octet][channel] in 16-byte chunks (the 8 tokens of one channel), with
+// one spare chunk after every 8 channels.  A fragment read (32 consecutive channels, one token octet)
+// is then a contiguous run of chunks, and the eight lanes that write the same channel-within-octet land
+// 9 chunks apart: both directions are free of bank conflicts.
+// The next stage's 16 loads per thread are in flight during the whole current stage.
+// =============================================================================================
+constexpr int T2 = 256;
+constexpr int KT2 = 64;                               // tokens per stage
+constexpr int OCT_CHUNKS = T2 + T2 / 8;               // chunks per token octet (with the spare ones)
+constexpr int OP_ELEMS = (KT2 / 8) * OCT_CHUNKS * 8;  // bf16 elements per operand tile
+constexpr size_t BIG_SMEM = (size_t)2 * 2 * OP_ELEMS * sizeof(uint16_t);
+
+__device__ __forceinline__ int chunk_of(int oct, int ch) { return oct * OCT_CHUNKS + ch + (ch >> 3); }
+
+// Tile order for the big kernel.  Upper-triangle tiles are enumerated super-tile by super-tile
+// (4 row tiles x 8 column tiles): the ~32 workgroups an XCD runs at any moment then touch about a dozen
+// distinct channel panels instead of ~30, so more of their loads hit that XCD's L2.
+__device__ __forceinline__ void blocked_tri_decode(int L, int T, int& tm, int& tn) {
+  constexpr int SM = 4, SN = 8;
+  int cum = 0;
+  for (int a = 0; a * SM < T; ++a) {
+    for (int b = (a * SM) / SN; b * SN < T; ++b) {
+      int cnt = 0;
+      for (int i = 0; i < SM; ++i) {
+        const int r = a * SM + i;
+        if (r >= T) break;
+        const int lo = max(r, b * SN), hi = min(T, b * SN + SN);
+        cnt += max(0, hi - lo);
+      }
+      if (L < cum + cnt) {
+        int k = L - cum;
+        for (int i = 0; i < SM; ++i) {
+          const int r = a * SM + i;
+          const int lo = max(r, b * SN), hi = min(T, b * SN + SN);
+          const int w = max(0, hi - lo);
+          if (k < w) {
+            tm = r;
+            tn = lo + k;
+            return;
+          }
+          k -= w;
+        }
+      }
+      cum += cnt;
+    }
+  }
+  tm = tn = 0;  // not reached for L < T(T+1)/2
+}
+
+struct Patch8 {
+  uint4 r[8];  // r[t] = 8 channels of token t0+t
+  // GUARD = false: the caller knows all 8 tokens and 8 channels are in range (no per-load branch)
+  template <bool GUARD>
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ X, long ldx, int t0, int tend, int c, int C) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (GUARD) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (t0 + i < tend && c < C) v = *reinterpret_cast<const uint4*>(X + (long)(t0 + i) * ldx + c);
+        r[i] = v;
+      } else {
+        r[i] = *reinterpret_cast<const uint4*>(X + (long)(t0 + i) * ldx + c);
+      }
+    }
+  }
+  // writes channel rows ch..ch+7 (ch a multiple of 8) of token octet `oct` of an operand tile
+  __device__ __forceinline__ void store(uint16_t* __restrict__ tile, int ch, int oct) const {
+    const uint32_t in[8][4] = {{r[0].x, r[0].y, r[0].z, r[0].w}, {r[1].x, r[1].y, r[1].z, r[1].w},
+                               {r[2].x, r[2].y, r[2].z, r[2].w}, {r[3].x, r[3].y, r[3].z, r[3].w},
+                               {r[4].x, r[4].y, r[4].z, r[4].w}, {r[5].x, r[5].y, r[5].z, r[5].w},
+                               {r[6].x, r[6].y, r[6].z, r[6].w}, {r[7].x, r[7].y, r[7].z, r[7].w}};
+    uint4* base = reinterpret_cast<uint4*>(tile) + chunk_of(oct, ch);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;  // high / low halves of a channel pair
+      uint4 o;
+      o.x = __builtin_amdgcn_perm(in[1][c >> 1], in[0][c >> 1], sel);
+      o.y = __builtin_amdgcn_perm(in[3][c >> 1], in[2][c >> 1], sel);
+      o.z = __builtin_amdgcn_perm(in[5][c >> 1], in[4][c >> 1], sel);
+      o.w = __builtin_amdgcn_perm(in[7][c >> 1], in[6][c >> 1], sel);
+      base[c] = o;
+    }
+  }
+};
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_big_kernel(
+    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
+    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint16_t* tiles = reinterpret_cast<uint16_t*>(smem);  // [stage][A,B][OP_ELEMS]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int L = xcd_remap(blockIdx.x, ntri * splits);
+  const int split = L / ntri;
+  int tm, tn;
+  blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
+  const int m0 = tm * T2, n0 = tn * T2;
+  const int tbeg = split * tokens_per_split;
+  const int tend = min(n, tbeg + tokens_per_split);
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // patches of this thread: waves 0,1 stage the A tile, waves 2,3 the B tile; token octets oct and oct+4
+  const int opnd = wave >> 1;
+  const int co = lane & 31;                         // channel octet
+  const int oct = ((wave & 1) << 1) | (lane >> 5);  // 0..3
+  const int cbase = (opnd ? n0 : m0) + 8 * co;
+  Patch8 p0, p1;
+  const int nk = (tend - tbeg + KT2 - 1) / KT2;
+  const bool interior = (m0 + T2 <= C) && (n0 + T2 <= C);  // wave-uniform: no channel of the tile is out of range
+  if (nk > 0) {
+    p0.load<true>(X, ldx, tbeg + 8 * oct, tend, cbase, C);
+    p1.load<true>(X, ldx, tbeg + 8 * (oct + 4), tend, cbase, C);
+    p0.store(tiles + opnd * OP_ELEMS, 8 * co, oct);
+    p1.store(tiles + opnd * OP_ELEMS, 8 * co, oct + 4);
+  }
+  __syncthreads();
+  const int lr = lane & 31, lk = lane >> 5;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+      const int t0 = tbeg + (kt + 1) * KT2;
+      if (interior && t0 + KT2 <= tend) {
+        p0.load<false>(X, ldx, t0 + 8 * oct, tend, cbase, C);
+        p1.load<false>(X, ldx, t0 + 8 * (oct + 4), tend, cbase, C);
+      } else {
+        p0.load<true>(X, ldx, t0 + 8 * oct, tend, cbase, C);
+        p1.load<true>(X, ldx, t0 + 8 * (oct + 4), tend, cbase, C);
+      }
+    }
+    const uint4* as = reinterpret_cast<const uint4*>(tiles + (cur * 2 + 0) * OP_ELEMS);
+    const uint4* bs = reinterpret_cast<const uint4*>(tiles + (cur * 2 + 1) * OP_ELEMS);
+    uint4 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      fa[0][i] = as[chunk_of(lk, wm * 128 + i * 32 + lr)];
+      fb[0][i] = bs[chunk_of(lk, wn * 128 + i * 32 + lr)];
+    }
+#pragma unroll
+    for (int kk = 0; kk < KT2 / 16; ++kk) {
+      if (kk + 1 < KT2 / 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          fa[(kk + 1) & 1][i] = as[chunk_of(2 * (kk + 1) + lk, wm * 128 + i * 32 + lr)];
+          fb[(kk + 1) & 1][i] = bs[chunk_of(2 * (kk + 1) + lk, wn * 128 + i * 32 + lr)];
+        }
+      }
+      // keep the fragment reads of the next step ahead of this step's MFMAs (the scheduler would
+      // otherwise sink each read to just before its first use and expose the LDS latency)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8n, fa[kk & 1][i]),
+                                                              __builtin_bit_cast(bf16x8n, fb[kk & 1][j]), acc[i][j], 0,
+                                                              0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt + 1 < nk) {
+      uint16_t* nx = tiles + ((cur ^ 1) * 2 + opnd) * OP_ELEMS;
+      p0.store(nx, 8 * co, oct);
+      p1.store(nx, 8 * co, oct + 4);
+    }
+    __syncthreads();
+  }
+
+  // epilogue straight from the accumulators: for a fixed register the 32 lanes of a half-wave cover
+  // 128 contiguous bytes of one row
+  const bool partial = splits > 1;
+  float* out = partial ? ws + ((long)split * ntri + (L - split * ntri)) * (T2 * T2) : H;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = wn * 128 + j * 32 + lr;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+        if (partial) {
+          out[r * T2 + c] = acc[i][j][v];
+        } else if (m0 + r < C && n0 + c < C) {
+          float* q = H + (long)(m0 + r) * ldh + n0 + c;
+          float val = alpha * acc[i][j][v];
+          if (beta != 0.f) val = fmaf(beta, *q, val);
+          *q = val;
+        }
+      }
+    }
+}
+
+// fixed-order sum of the split partials of the big kernel; upper tiles only
+__global__ __launch_bounds__(256) void syrk_big_reduce_kernel(float* __restrict__ H, long ldh, int C, float alpha,
+                                                              float beta, int ntri, int splits,
+                                                              const float* __restrict__ ws) {
+  const int L = blockIdx.y;
+  int tm, tn;
+  blocked_tri_decode(L, (C + T2 - 1) / T2, tm, tn);
+  const int idx = blockIdx.x * 256 + threadIdx.x;  // one float4 of the tile
+  const int r = idx >> 6, c = (idx & 63) << 2;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < splits; ++k) {
+    const float4 v = *reinterpret_cast<const float4*>(ws + ((long)k * ntri + L) * (T2 * T2) + r * T2 + c);
+    s.x += v.x;
+    s.y += v.y;
+    s.z += v.z;
+    s.w += v.w;
+  }
+  const float e[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int gr = tm * T2 + r, gc = tn * T2 + c + q;
+    if (gr < C && gc < C) {
+      float* p = H + (long)gr * ldh + gc;
+      float val = alpha * e[q];
+      if (beta != 0.f) val = fmaf(beta, *p, val);
+      *p = val;
+    }
+  }
+}
+
+// lower triangle <- transpose of the upper triangle, 64x64 tiles through LDS
+__global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, long ldh, int C) {
+  __shared__ float t[64][65];
+  int bi, bj;
+  tri_decode(blockIdx.x, bi, bj);  // bi <= bj: source tile rows bi, cols bj
+  if (bi == bj) {
+    for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
+      if (c > r && bi * 64 + c < C) t[r][c] = H[(long)(bi * 64 + r) * ldh + bi * 64 + c];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+      const int r = idx >> 6, c = idx & 63;
+      if (c < r && bi * 64 + r < C) H[(long)(bi * 64 + r) * ldh + bi * 64 + c] = t[c][r];
+    }
+    return;
+  }
+  for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+    const int r = idx >> 6, c = idx & 63;
+    if (bi * 64 + r < C && bj * 64 + c < C) t[r][c] = H[(long)(bi * 64 + r) * ldh + bj * 64 + c];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 64 * 64; idx += 256) {
+    const int r = idx >> 6, c = idx & 63;  // destination row bj*64+r, col bi*64+c
+    if (bj * 64 + r < C && bi * 64 + c < C) H[(long)(bj * 64 + r) * ldh + bi * 64 + c] = t[c][r];
+  }
+}
+
+void pick_split_big(int n, int C, int& ntri, int& splits, int& tps) {
+  const int tiles = (C + T2 - 1) / T2;
+  ntri = tiles * (tiles + 1) / 2;
+  splits = 1;
+  if (ntri < 224) splits = (256 + ntri - 1) / ntri;  // one workgroup per CU is the most this kernel runs
+  const int max_splits = (n + 2047) / 2048;          // at least 2048 tokens per split
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 64) splits = 64;
+  if (splits < 1) splits = 1;
+  tps = (n + splits - 1) / splits;
+  tps = (tps + KT2 - 1) / KT2 * KT2;
+  splits = (n + tps - 1) / tps;
+  if (splits < 1) splits = 1;
+}
+
+bool use_big(const void* X, long ldx, int n, int C) {
+  return n >= 256 && C >= 256 && (C % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
+}
+
 constexpr size_t SMEM_BYTES = (size_t)T * EPI_LD * sizeof(float);  // 66048 >= 4*TILE_ELEMS*2 = 40960
 
 void pick_split(int n, int C, int& ntri, int& splits, int& tps) {
@@ -215,7 +499,17 @@ extern "C" size_t mq_hessian_syrk_workspace_bytes(int n, int C) {
   if (n <= 0 || C <= 0) return 0;
   int ntri, splits, tps;
   pick_split(n, C, ntri, splits, tps);
-  return splits > 1 ? (size_t)splits * ntri * T * T * sizeof(float) : 0;
+  const size_t small = splits > 1 ? (size_t)splits * ntri * T * T * sizeof(float) : 0;
+  pick_split_big(n, C, ntri, splits, tps);
+  const size_t big = splits > 1 ? (size_t)splits * ntri * T2 * T2 * sizeof(float) : 0;
+  return small > big ? small : big;  // either kernel may be chosen, depending on alignment
+}
+
+extern "C" int mq_symmetrize_upper(float* H, long ldh, int C, void* stream) {
+  if (!H || C <= 0 || ldh < C) return MQ_ERR_ARG;
+  const int t = (C + 63) / 64;
+  hipLaunchKernelGGL(symmetrize_kernel, dim3(t * (t + 1) / 2), dim3(256), 0, (hipStream_t)stream, H, ldh, C);
+  return mq_check_launch();
 }
 
 extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
@@ -223,8 +517,31 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
   if (!H || C <= 0 || n < 0 || ldh < C || (n > 0 && (!X || ldx < C))) return MQ_ERR_ARG;
   if ((C & 1) || (ldx & 1) || ((uintptr_t)X & 3)) return MQ_ERR_ARG;  // 4-byte channel-pair loads
   int ntri, splits, tps;
-  pick_split(n > 0 ? n : 1, C, ntri, splits, tps);
   hipStream_t st = (hipStream_t)stream;
+  if (n > 0 && use_big(X, ldx, n, C)) {
+    pick_split_big(n, C, ntri, splits, tps);
+    if (splits > 1) {
+      const size_t need = (size_t)splits * ntri * T2 * T2 * sizeof(float);
+      if (!workspace || workspace_bytes < need) return MQ_ERR_WORKSPACE;
+    }
+    static bool big_attr = false;
+    if (!big_attr) {
+      (void)hipFuncSetAttribute((const void*)syrk_bf16_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)BIG_SMEM);
+      big_attr = true;
+    }
+    hipLaunchKernelGGL(syrk_bf16_big_kernel, dim3(ntri * splits), dim3(256), BIG_SMEM, st, H, ldh, (const uint16_t*)X,
+                       ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    int rc = mq_check_launch();
+    if (rc != MQ_OK) return rc;
+    if (splits > 1) {
+      hipLaunchKernelGGL(syrk_big_reduce_kernel, dim3(T2 * T2 / 4 / 256, ntri), dim3(256), 0, st, H, ldh, C, alpha, beta,
+                         ntri, splits, (const float*)workspace);
+      if ((rc = mq_check_launch()) != MQ_OK) return rc;
+    }
+    return mirror ? mq_symmetrize_upper(H, ldh, C, stream) : MQ_OK;
+  }
+  pick_split(n > 0 ? n : 1, C, ntri, splits, tps);
   static bool attr_done = false;
   if (!attr_done) {
     (void)hipFuncSetAttribute((const void*)syrk_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);

@@ -88,7 +88,9 @@ class GPTQ:
             return  # the reference would divide 0/0 here when nothing was collected before
         beta = self.num_samples / (self.num_samples + num_new_samples)
         alpha = 2.0 / (self.num_samples + num_new_samples)
-        ops.hessian_syrk_(self.H, input, beta, alpha, mirror=True)
+        # only the upper triangle is accumulated; quantization_pre_step mirrors it once
+        ops.hessian_syrk_(self.H, input, beta, alpha, mirror=False)
+        self._H_upper_only = True
         self.num_samples += num_new_samples
 
     add_batch = update
@@ -115,8 +117,15 @@ class GPTQ:
         torch.cuda.empty_cache()
 
     # ---- pre-step: src/gptq.py:122-154 --------------------------------------------------------------
+    def symmetrize_hessian(self) -> None:
+        """`update` maintains the upper triangle of H only; this mirrors it onto the lower one."""
+        if self.H is not None and getattr(self, "_H_upper_only", False):
+            ops.symmetrize_upper_(self.H)
+            self._H_upper_only = False
+
     @torch.no_grad()
     def quantization_pre_step(self) -> None:
+        self.symmetrize_hessian()
         if self.H is None:
             if self.tied_gptq_handle:
                 self.H = self.tied_gptq_handle.H

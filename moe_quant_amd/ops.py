@@ -77,6 +77,17 @@ def hessian_syrk_(H: Tensor, X: Tensor, beta: float, alpha: float, mirror: bool 
     return H
 
 
+def symmetrize_upper_(H: Tensor) -> Tensor:
+    """Copies the upper triangle of H onto the lower one, in place."""
+    _dev(H)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    check(lib.mq_symmetrize_upper(H.data_ptr(), H.stride(0), C, _stream(H)), "mq_symmetrize_upper")
+    return H
+
+
 # ---- (2) factorisation -------------------------------------------------------------------------------
 def factor_upper_inverse_(A: Tensor, info: Optional[Tensor] = None, normalize: bool = True) -> Tensor:
     """In place A -> upper U = chol(A^-1, upper), rows scaled to unit diagonal when `normalize`.

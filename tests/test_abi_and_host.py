@@ -66,9 +66,9 @@ def test_pure_size_query_needs_no_gpu():
     from moe_quant_amd import _lib
 
     lib = _lib.load()
-    assert lib.mq_hessian_syrk_workspace_bytes(8192, 7168) == 0  # 1596 tiles fill the GPU: no split
-    need = lib.mq_hessian_syrk_workspace_bytes(65536, 2048)  # 136 tiles: token range is split
-    assert need > 0 and need % (136 * 128 * 128 * 4) == 0
+    assert lib.mq_hessian_syrk_workspace_bytes(8192, 7168) == 0  # enough tiles to fill the GPU: no split
+    need = lib.mq_hessian_syrk_workspace_bytes(65536, 2048)  # 36 tiles of 256x256: the token range is split
+    assert need > 0 and need % (36 * 256 * 256 * 4) == 0
     assert lib.mq_hessian_syrk_workspace_bytes(0, 128) == 0
 
 

@@ -50,6 +50,7 @@ def test_hip_path_reproduces_golden(dev, tag, order):
     h = GPTQ(layer, group_size=128, sym=True, rel_damp=0.01, block_size=128, quantization_order=order)
     h.update(X[:100].to(dev))
     h.update(X[100:].to(dev))
+    h.symmetrize_hessian()
     _check_H(h.H.cpu(), 1e-5)
     q, s, z = h.quantize(4)
     assert np.array_equal(s.cpu().view(torch.int16).numpy(), G[f"scale_bits_{tag}"])

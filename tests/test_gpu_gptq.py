@@ -37,6 +37,7 @@ def _run_case(case, dev, chunks=3, code_gate=0.999):
         Href, n = O.hessian_update(Href, n, x)
     assert h.tokens_collected == case.X.shape[0] == n
     H64 = O.hessian_fp64([case.X])
+    h.symmetrize_hessian()
     herr = ((h.H.cpu().double() - H64).norm() / H64.norm()).item()
     q, s, z = h.quantize(4)
     ref = O.quantize_linear(case.W, Href.clone(), group_size=case.group_size, rel_damp=case.rel_damp,
@@ -96,6 +97,7 @@ def test_nan_hessian_falls_back(dev):
     W = synth.weight(64, 256, 2)
     h = GPTQ(_layer(W, dev), 128, True)
     h.update(synth.activations_outlier(300, 256, 3).to(dev))
+    h.symmetrize_hessian()
     h.H[3, 7] = float("nan")
     q, s, z = h.quantize(4)
     assert h.issue_nan_hessian

@@ -96,14 +96,17 @@ def test_hessian_running_mean_matches_oracle(dev):
 
 
 def test_hessian_upper_only(dev):
-    C, n = 256, 512
+    C, n = 512, 512
     X = synth.activations_outlier(n, C, seed=3).to(dev)
     H = torch.full((C, C), 7.0, device=dev)
     ops.hessian_syrk_(H, X, 0.0, 1.0, mirror=False)
     Hc = H.cpu()
     ref = (X.cpu().double().t() @ X.cpu().double())
     assert (torch.triu(Hc).double() - torch.triu(ref)).abs().max() / ref.abs().max() < 1e-5
-    assert torch.all(Hc[128:, :128] == 7.0)  # strictly-lower off-diagonal tile untouched
+    assert torch.all(Hc[256:, :256] == 7.0)  # below the diagonal tiles nothing is written
+    ops.symmetrize_upper_(H)
+    Hc = H.cpu()
+    assert torch.equal(Hc, Hc.t()) and (Hc.double() - ref).abs().max() / ref.abs().max() < 1e-5
 
 
 # ---------------------------------------------------------------- (2) factorisation
