@@ -30,7 +30,87 @@ def parse():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
+    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer"],
+                    help="config1 (default, the benchmark line) or moe_layer (config 3: whole MoE layer, one pass)")
+    ap.add_argument("--experts", type=int, default=256)
+    ap.add_argument("--tokens", type=int, default=2_097_152)
+    ap.add_argument("--check-experts", type=int, default=2, help="moe_layer: experts compared with the CPU oracle")
     return ap.parse_args()
+
+
+def moe_layer_main(args):
+    """Config 3: every Hessian of a DeepSeek-V3-shaped MoE layer accumulated, 3 linears per expert quantized
+    and packed, on one GPU.  Prints one JSON line (metric: MoE-layer wall seconds)."""
+    import torch
+
+    from moe_quant_amd import _lib, synth
+    from moe_quant_amd.moe_layer import ExpertWeights, quantize_moe_layer
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    t0 = time.perf_counter()
+    x, ids, ex = synth.moe_layer_on_device(dev, args.experts, args.tokens)
+    torch.cuda.synchronize()
+    t_gen = time.perf_counter() - t0
+    experts = [ExpertWeights(*w) for w in ex]
+    # warm-up on a tiny problem so that one-time costs (module load, allocator growth) stay out of the clock
+    quantize_moe_layer(x[:4096], ids[:4096] % 2, experts[:2])
+    counts = torch.bincount(ids.flatten(), minlength=args.experts)
+    check = torch.argsort(counts, descending=True)[: args.check_experts].tolist() if args.check_experts else []
+    res = quantize_moe_layer(x, ids, experts, keep_codes=check)
+    C, I = x.shape[1], experts[0].gate.shape[0]
+    n_e = torch.tensor(res.tokens_per_expert, dtype=torch.float64)
+    flop_syrk = float((n_e * (C * (C + 1) + I * (I + 1))).sum())
+    out = {
+        "metric": "MoE-layer wall seconds (256 experts x 3 linears, 2M routed calibration tokens)",
+        "value": round(res.seconds["total"], 3),
+        "unit": "s",
+        "n_gpus": 1,
+        "steps": 1,
+        "warmup": 0,
+        "ms_per_step": round(res.seconds["total"] * 1e3, 1),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "config 3: DeepSeek-V3-shaped MoE layer, all Hessians resident, GPTQ 4-bit g128 on all linears",
+                   "experts": args.experts, "tokens": args.tokens, "top_k": int(ids.shape[1]), "hidden": C, "inter": I,
+                   "linears": 3 * args.experts},
+        "seconds": {k: round(v, 3) for k, v in res.seconds.items()},
+        "generate_inputs_s": round(t_gen, 2),
+        "tokens_per_expert": {"min": int(n_e.min()), "max": int(n_e.max()), "mean": float(n_e.mean())},
+        "hessian_algorithmic_tflop": round(flop_syrk / 1e12, 1),
+        "issues": res.issues,
+        "note": "hessians_incl_gather_and_forward counts the per-expert token gather and the expert forward "
+                "(two bf16 matmuls + SiLU product, torch) that produce the down-projection inputs",
+    }
+    if check and not args.no_cpu_baseline:
+        from oracle import gptq_oracle as O
+
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        par = {}
+        t_cpu = 0.0
+        for e in check:
+            for proj, w in (("gate_proj", experts[e].gate), ("down_proj", experts[e].down)):
+                Hc = res.hessians[f"{e}.{proj}"].cpu()
+                tc = time.perf_counter()
+                ref = O.quantize_linear(w.cpu(), Hc)
+                t_cpu += time.perf_counter() - tc
+                q = res.qweight[f"{e}.{proj}"].cpu()
+                par[f"{e}.{proj}"] = {
+                    "code_match": round((q == ref["qweight"]).float().mean().item(), 6),
+                    "scales_equal": bool(torch.equal(res.scales[f"{e}.{proj}"].cpu(), ref["scale"])),
+                }
+        out["parity_vs_cpu_oracle"] = par
+        out["cpu_baseline"] = {
+            "value": round(t_cpu / (2 * len(check)), 3), "unit": "s per linear (quantize only, Hessian given)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{2 * len(check)} linears of the layer (gate and down of the {len(check)} busiest experts), "
+                      f"extrapolated layer quantize time = {t_cpu / (2 * len(check)) * 3 * args.experts:.0f} s",
+        }
+    print(json.dumps(out))
 
 
 def main():
@@ -38,6 +118,8 @@ def main():
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU (no sharding, no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "moe_layer":
+        return moe_layer_main(args)
     import torch
 
     from moe_quant_amd import _lib, ops, synth

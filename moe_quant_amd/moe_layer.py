@@ -1,0 +1,134 @@
+"""One MoE layer through the engine on one GPU: the expert part of MoE-Quant's per-block flow
+(quant.py:241-411) with the model forward replaced by its two ingredients the Hessians need --
+the routed token sets and the SwiGLU product that feeds each down projection.
+
+Flow, as in the reference: all Hessians of the block are collected first (gate and up of an expert
+share one, quant.py:258-277), then every linear is quantized and packed.  Everything stays resident
+in HBM: 256 x 7168^2 fp32 gate/up Hessians (52.6 GB) + 256 x 2048^2 (4.3 GB) + 2M x 7168 bf16 tokens
+(30 GB) + bf16 weights (22.5 GB) fit one MI355X.  Routed activations are gathered one expert at a time
+(materialising all top-8 copies at once would take 240 GB).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+import torch.nn as nn
+
+from .gptq import GPTQ
+
+
+@dataclass
+class ExpertWeights:
+    gate: torch.Tensor  # (I, C) bf16
+    up: torch.Tensor  # (I, C) bf16
+    down: torch.Tensor  # (C, I) bf16
+
+
+@dataclass
+class LayerResult:
+    seconds: Dict[str, float] = field(default_factory=dict)
+    tokens_per_expert: List[int] = field(default_factory=list)
+    packed: Dict[str, torch.Tensor] = field(default_factory=dict)  # "<e>.<proj>" -> int32 words (kept if asked)
+    scales: Dict[str, torch.Tensor] = field(default_factory=dict)
+    qweight: Dict[str, torch.Tensor] = field(default_factory=dict)  # only for the experts listed in keep_codes
+    hessians: Dict[str, torch.Tensor] = field(default_factory=dict)  # idem (undamped copies)
+    issues: Dict[str, int] = field(default_factory=dict)
+
+
+def route_tokens(expert_ids: torch.Tensor, n_experts: int):
+    """expert_ids (T, top_k) -> (order, offsets): order[offsets[e]:offsets[e+1]] are the token rows of expert e."""
+    flat = expert_ids.reshape(-1)
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=n_experts)
+    offsets = torch.zeros(n_experts + 1, dtype=torch.int64, device=flat.device)
+    offsets[1:] = torch.cumsum(counts, 0)
+    return order // expert_ids.shape[1], offsets.tolist()
+
+
+@torch.no_grad()
+def quantize_moe_layer(
+    x: torch.Tensor,
+    expert_ids: torch.Tensor,
+    experts: List[ExpertWeights],
+    bits: int = 4,
+    group_size: int = 128,
+    rel_damp: float = 0.01,
+    block_size: int = 128,
+    keep_outputs: bool = False,
+    keep_codes: Optional[List[int]] = None,
+    max_rows_per_update: int = 1 << 17,
+) -> LayerResult:
+    """x (T, C) bf16 on the GPU, expert_ids (T, top_k) int64 on the GPU."""
+    dev = x.device
+    E = len(experts)
+    keep_codes = set(keep_codes or [])
+    res = LayerResult()
+    sync = lambda: torch.cuda.synchronize(dev)
+
+    def linear(w):
+        m = nn.Linear(w.shape[1], w.shape[0], bias=False, dtype=w.dtype, device=dev)
+        m.weight.data = w
+        return m
+
+    handles = []
+    for ew in experts:
+        g = GPTQ(linear(ew.gate), group_size, True, rel_damp, block_size)
+        u = GPTQ(linear(ew.up), group_size, True, rel_damp, block_size, tied_gptq_handle=g)
+        d = GPTQ(linear(ew.down), group_size, True, rel_damp, block_size)
+        handles.append((g, u, d))
+
+    # ---- phase 1: Hessians of the whole block
+    sync()
+    t0 = time.perf_counter()
+    rows, offsets = route_tokens(expert_ids, E)
+    sync()
+    res.seconds["route"] = time.perf_counter() - t0
+    t_gather = t_fwd = 0.0
+    t1 = time.perf_counter()
+    for e, (g, u, d) in enumerate(handles):
+        lo, hi = offsets[e], offsets[e + 1]
+        res.tokens_per_expert.append(hi - lo)
+        for s in range(lo, hi, max_rows_per_update):
+            idx = rows[s : min(hi, s + max_rows_per_update)]
+            xe = x.index_select(0, idx)  # (n, C) bf16
+            g.update(xe)
+            a = torch.nn.functional.silu(xe @ experts[e].gate.t()) * (xe @ experts[e].up.t())  # the expert's forward
+            d.update(a)
+    sync()
+    res.seconds["hessians_incl_gather_and_forward"] = time.perf_counter() - t1
+
+    # ---- phase 2: quantize + pack 3 linears per expert
+    t2 = time.perf_counter()
+    issues = {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
+    for e, (g, u, d) in enumerate(handles):
+        if e in keep_codes:
+            g.symmetrize_hessian()
+            d.symmetrize_hessian()
+            if g.H is not None:
+                res.hessians[f"{e}.gate_proj"] = g.H.clone()
+            if d.H is not None:
+                res.hessians[f"{e}.down_proj"] = d.H.clone()
+        for name, h in (("gate_proj", g), ("up_proj", u), ("down_proj", d)):
+            q, s, z = h.quantize(bits)
+            words = h.packed_words()
+            issues["zero_samples"] += int(h.issue_zero_samples)
+            issues["nan_hessian"] += int(h.issue_nan_hessian)
+            issues["non_invertible"] += int(h.issue_non_invertible)
+            if keep_outputs:
+                res.packed[f"{e}.{name}"] = words
+                res.scales[f"{e}.{name}"] = s
+            if e in keep_codes:
+                res.qweight[f"{e}.{name}"] = q
+                res.scales[f"{e}.{name}"] = s
+        for h in (g, u, d):  # as quant.py:330: free per-linear state as soon as the linear is done
+            h.H = None
+            h._hessian_inv = None
+            h.W = h.layer.weight
+    sync()
+    res.seconds["quantize_and_pack"] = time.perf_counter() - t2
+    res.seconds["total"] = time.perf_counter() - t0
+    res.issues = issues
+    return res

@@ -117,3 +117,38 @@ def moe_routing(n_tokens: int, n_experts: int = 256, top_k: int = 8, seed: int =
         ids[s:e] = torch.topk(torch.softmax(logits, -1), top_k, dim=-1).indices
     counts = torch.bincount(ids.flatten(), minlength=n_experts)
     return ids, counts
+
+
+def moe_layer_on_device(device, n_experts: int = 256, tokens: int = 2_097_152, hidden: int = 7168,
+                        inter: int = 2048, top_k: int = 8, seed: int = 300, zipf_s: float = 1.1):
+    """Config 3 generated directly in HBM (30 GB of tokens would take minutes over PCIe): returns
+    (x (T, hidden) bf16, expert_ids (T, top_k) int64, [(gate, up, down) bf16]).  Same distributions as
+    the CPU generators; seeded with a device generator, so bits are reproducible per device type."""
+    import torch
+
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    x = torch.empty(tokens, hidden, dtype=torch.bfloat16, device=device)
+    outl = outlier_channels(hidden, seed + 1).to(device)
+    step = 1 << 16
+    for s in range(0, tokens, step):
+        e = min(tokens, s + step)
+        blk = torch.randn(e - s, hidden, generator=g, device=device)
+        blk[:, outl] *= 20.0
+        x[s:e] = blk.to(torch.bfloat16)
+    ranks = torch.randperm(n_experts, generator=_gen(seed + 2)).float() + 1.0
+    bias = -zipf_s * torch.log(ranks)
+    bias = (bias - bias.mean()).to(device)
+    ids = torch.empty(tokens, top_k, dtype=torch.int64, device=device)
+    step = 1 << 18
+    for s in range(0, tokens, step):
+        e = min(tokens, s + step)
+        logits = torch.randn(e - s, n_experts, generator=g, device=device) + bias
+        ids[s:e] = torch.topk(torch.softmax(logits, -1), top_k, dim=-1).indices
+    experts = []
+    for _ in range(n_experts):
+        gate = (torch.randn(inter, hidden, generator=g, device=device) * 0.02).to(torch.bfloat16)
+        up = (torch.randn(inter, hidden, generator=g, device=device) * 0.02).to(torch.bfloat16)
+        down = (torch.randn(hidden, inter, generator=g, device=device) * 0.02).to(torch.bfloat16)
+        experts.append((gate, up, down))
+    return x, ids, experts
