@@ -210,14 +210,20 @@ def main():
     }
     # dominant kernel of the step: the factorisation chain (fp32 MFMA bound); achieved = algorithmic
     # (2/3) C^3 flop / measured device time of the chain
+    # HBM bytes per factorisation of a 7168^2 matrix, from the two rocprofv3 --pmc runs summarised in
+    # profiles/config1_bench_hbm_traffic.md (2.00*FETCH_SIZE + 1.00*WRITE_SIZE, calibrated on copy/fill kernels)
+    traffic = 7.79e9 if C == 7168 else None
     roofline = {
-        "kernel": "factorisation chain (revchol_diag + gemm_f32 panel/trailing/triangular-inverse)",
+        "kernel": "mq_factor_upper_inverse = trail_diag_kernel + gemm_f32_kernel<true,true>/<false,true> + "
+                  "revchol_diag_kernel + unit_diag_kernel (one launch sequence per call; largest share of the step)",
         "bound": "mfma",
         "achieved": round(flop_factor / t_factor / 1e9, 3),
         "peak": PEAK_FP32_MFMA,
         "unit": "TFLOP/s",
         "frac": round(flop_factor / t_factor / 1e9 / PEAK_FP32_MFMA, 4),
-        "traffic": None,
+        "traffic": traffic,
+        "algorithmic_flop_per_launch": flop_factor,
+        "ms_per_launch": round(t_factor, 4),
     }
 
     cpu = None
