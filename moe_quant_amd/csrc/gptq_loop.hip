@@ -50,57 +50,56 @@ constexpr int UL = 132;      // pitch of the U block in LDS (16-byte aligned row
 
 typedef const int __attribute__((address_space(4))) * cint_p;  // constant address space: scalar loads
 
-// One wavefront owns 64 rows.  The 128-column block of those rows sits in LDS ([column][lane], so
-// every access is conflict-free) next to the 128x128 block of U.  16 columns at a time move to
-// registers for the strictly sequential part; their 16 errors are then folded into the rest of the
-// block, 16 columns per pass.  The multipliers U[j,k] are the same for every lane: they are read from
-// LDS with all lanes on one address (a broadcast, four values per read).  For every weight the updates
-// are applied in ascending j with one fma each, exactly the order of the sequential reference.
+// One workgroup (four wavefronts) owns 64 rows; lane l of every wavefront is row l.  The 128-column
+// block of those rows sits in LDS ([column][lane], so every access is conflict-free) next to the
+// 128x128 block of U.  16 columns at a time move to the registers of wavefront 0 for the strictly
+// sequential part; their 16 errors are published in LDS and all four wavefronts fold them into the rest
+// of the block, each taking every fourth pass of 16 columns.  The multipliers U[j,k] are the same for
+// every lane: they are read from LDS with all lanes on one address (a broadcast, four values per read).
+// For every weight the updates are applied in ascending j with one fma each, exactly the order of the
+// sequential reference.
 //
-// A lone wavefront per CU cannot hide latency by switching waves, so every phase issues its loads in
-// bulk before the first use: the kernel is built from branch-free unrolled blocks for that reason
-// (ROWMAP / QZERO are template flags, the rounding mode is a select).
+// Nothing else runs on the CU to hide latency, so every phase issues its loads in bulk before the first
+// use: the kernel is built from branch-free unrolled blocks for that reason (ROWMAP / QZERO are template
+// flags, the rounding mode is a select).
 template <bool FULL, bool ROWMAP, bool QZERO>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void gptq_block_kernel(LoopArgs a, int i1,
-                                                                                                  int nb) {
-  __shared__ __attribute__((aligned(16))) float tile[B * WSTRIDE];
-  __shared__ __attribute__((aligned(16))) float ut[B * UL];
-  const int lane = threadIdx.x;
+__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int nb) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* tile = reinterpret_cast<float*>(smem);  // [B][WSTRIDE]
+  float* ut = tile + B * WSTRIDE;                // [B][UL]
+  float* esh = ut + B * UL;                      // [MB][WSTRIDE] errors of the current micro-block
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r0 = blockIdx.x * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
   // does, so no branch in this kernel ever diverges.
   const int r = min(r0 + lane, a.R - 1);
   float* __restrict__ wp = a.Wt + (long)i1 * a.ldw + r;
+  {
+    float t[32];  // each wavefront stages 32 of the 128 columns
 #pragma unroll
-  for (int kb = 0; kb < B; kb += 32) {
-    float t[32];
+    for (int k = 0; k < 32; ++k) t[k] = (FULL || wave * 32 + k < nb) ? wp[(long)(wave * 32 + k) * a.ldw] : 0.f;
 #pragma unroll
-    for (int k = 0; k < 32; ++k) t[k] = (FULL || kb + k < nb) ? wp[(long)(kb + k) * a.ldw] : 0.f;
-#pragma unroll
-    for (int k = 0; k < 32; ++k) tile[(kb + k) * WSTRIDE + lane] = t[k];
+    for (int k = 0; k < 32; ++k) tile[(wave * 32 + k) * WSTRIDE + lane] = t[k];
   }
   {
     const float* __restrict__ Ub = a.U + (long)i1 * a.ldu + i1;
     const bool vec = FULL && ((a.ldu & 3) == 0) && ((((uintptr_t)Ub) & 15) == 0);
     if (vec) {
+      float4 v[16];
 #pragma unroll
-      for (int it = 0; it < B * (B / 4) / 64; it += 16) {
-        float4 v[16];
+      for (int u = 0; u < 16; ++u) {
+        const int idx = tid + u * 256;
+        const int j = idx >> 5, k = (idx & 31) << 2;
+        v[u] = (k + 3 > j) ? *reinterpret_cast<const float4*>(Ub + (long)j * a.ldu + k) : make_float4(0, 0, 0, 0);
+      }
 #pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          const int idx = lane + (it + u) * 64;
-          const int j = idx >> 5, k = (idx & 31) << 2;
-          v[u] = (k + 3 > j) ? *reinterpret_cast<const float4*>(Ub + (long)j * a.ldu + k) : make_float4(0, 0, 0, 0);
-        }
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          const int idx = lane + (it + u) * 64;
-          const int j = idx >> 5, k = (idx & 31) << 2;
-          *reinterpret_cast<float4*>(&ut[j * UL + k]) = v[u];
-        }
+      for (int u = 0; u < 16; ++u) {
+        const int idx = tid + u * 256;
+        const int j = idx >> 5, k = (idx & 31) << 2;
+        *reinterpret_cast<float4*>(&ut[j * UL + k]) = v[u];
       }
     } else {
-      for (int idx = lane; idx < B * B; idx += 64) {
+      for (int idx = tid; idx < B * B; idx += 256) {
         const int j = idx >> 7, k = idx & 127;
         ut[j * UL + k] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
       }
@@ -113,94 +112,114 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 1))) void
   cint_p srp = (cint_p)(a.scale_row);
 #pragma unroll 1
   for (int c0 = 0; c0 < cend; c0 += MB) {
-    float w[MB], e[MB], sc[MB], zz[MB];
-    float4 um[MB][MB / 4];
+    if (wave == 0) {
+      float w[MB], e[MB], sc[MB], zz[MB];
+      float4 um[MB][MB / 4];
 #pragma unroll
-    for (int t = 0; t < MB; ++t) {
-      const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
-      const int srow = ROWMAP ? srp[col] : col;
-      sc[t] = a.scale[(long)srow * a.lds + r];
-      zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
-      w[t] = tile[(c0 + t) * WSTRIDE + lane];
-    }
-#pragma unroll
-    for (int J = 0; J < MB; ++J)
-#pragma unroll
-      for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
-        um[J][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + J) * UL + c0 + 4 * t4]);
-#pragma unroll
-    for (int J = 0; J < MB; ++J) {
-      const float s = sc[J], z = zz[J];
-      const float x = w[J];
-      const float v = x / s + z;
-      float q = floorf(v + 0.5f);
-      q = fminf(fmaxf(q, 0.f), maxq);
-      const float y = round_dtype((q - z) * s, rd);
-      e[J] = (FULL || c0 + J < nb) ? (y - x) : 0.f;
-      if (FULL || c0 + J < nb) {
-        wp[(long)(c0 + J) * a.ldw] = y;
-        a.Qt[(long)(i1 + c0 + J) * a.R + r] = (uint8_t)q;
-        a.E[(long)(c0 + J) * a.R + r] = e[J];
+      for (int t = 0; t < MB; ++t) {
+        const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
+        const int srow = ROWMAP ? srp[col] : col;
+        sc[t] = a.scale[(long)srow * a.lds + r];
+        zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
+        w[t] = tile[(c0 + t) * WSTRIDE + lane];
       }
 #pragma unroll
-      for (int t = J + 1; t < MB; ++t) {
-        const float4 u4 = um[J][t >> 2];
-        const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
-        w[t] = fmaf(u, e[J], w[t]);
-      }
-    }
-    // fold the 16 errors into the remaining columns of the block, 16 columns per pass; U rows are
-    // fetched four at a time, one group ahead of the FMAs that consume them
-#pragma unroll 1
-    for (int k0 = c0 + MB; k0 < cend; k0 += MB) {
-      float x[MB];
-      float4 ug[2][4][MB / 4];
+      for (int J = 0; J < MB; ++J)
 #pragma unroll
-      for (int t = 0; t < MB; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
+        for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
+          um[J][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + J) * UL + c0 + 4 * t4]);
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int t4 = 0; t4 < MB / 4; ++t4)
-          ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + jj) * UL + k0 + 4 * t4]);
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        if (g < 3) {
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-            for (int t4 = 0; t4 < MB / 4; ++t4)
-              ug[(g + 1) & 1][jj][t4] =
-                  *reinterpret_cast<const float4*>(&ut[(c0 + 4 * (g + 1) + jj) * UL + k0 + 4 * t4]);
+      for (int J = 0; J < MB; ++J) {
+        const float s = sc[J], z = zz[J];
+        const float x = w[J];
+        const float v = x / s + z;
+        float q = floorf(v + 0.5f);
+        q = fminf(fmaxf(q, 0.f), maxq);
+        const float y = round_dtype((q - z) * s, rd);
+        e[J] = (FULL || c0 + J < nb) ? (y - x) : 0.f;
+        esh[J * WSTRIDE + lane] = e[J];
+        if (FULL || c0 + J < nb) {
+          wp[(long)(c0 + J) * a.ldw] = y;
+          a.Qt[(long)(i1 + c0 + J) * a.R + r] = (uint8_t)q;
+          a.E[(long)(c0 + J) * a.R + r] = e[J];
         }
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const float ej = e[4 * g + jj];
+        for (int t = J + 1; t < MB; ++t) {
+          const float4 u4 = um[J][t >> 2];
+          const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
+          w[t] = fmaf(u, e[J], w[t]);
+        }
+      }
+    }
+    __syncthreads();
+    // fold the 16 errors into the remaining columns of the block, 16 columns per pass, passes dealt
+    // round-robin to the four wavefronts; U rows are fetched four at a time, one group ahead of the FMAs
+    if (c0 + MB + MB * wave < cend) {
+      float e[MB];
 #pragma unroll
-          for (int t4 = 0; t4 < MB / 4; ++t4) {
-            const float4 u = ug[g & 1][jj][t4];
-            x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
-            x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
-            x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
-            x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
+      for (int J = 0; J < MB; ++J) e[J] = esh[J * WSTRIDE + lane];
+#pragma unroll 1
+      for (int k0 = c0 + MB + MB * wave; k0 < cend; k0 += 4 * MB) {
+        float x[MB];
+        float4 ug[2][4][MB / 4];
+#pragma unroll
+        for (int t = 0; t < MB; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+          for (int t4 = 0; t4 < MB / 4; ++t4)
+            ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + jj) * UL + k0 + 4 * t4]);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          if (g < 3) {
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+              for (int t4 = 0; t4 < MB / 4; ++t4)
+                ug[(g + 1) & 1][jj][t4] =
+                    *reinterpret_cast<const float4*>(&ut[(c0 + 4 * (g + 1) + jj) * UL + k0 + 4 * t4]);
+          }
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            const float ej = e[4 * g + jj];
+#pragma unroll
+            for (int t4 = 0; t4 < MB / 4; ++t4) {
+              const float4 u = ug[g & 1][jj][t4];
+              x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
+              x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
+              x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
+              x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
+            }
           }
         }
-      }
 #pragma unroll
-      for (int t = 0; t < MB; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
+        for (int t = 0; t < MB; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
+      }
     }
+    __syncthreads();
   }
 }
+
+constexpr size_t BLOCK_SMEM = (size_t)(B * WSTRIDE + B * UL + MB * WSTRIDE) * sizeof(float);
 
 template <bool ROWMAP, bool QZERO>
 int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   const int grid = (a.R + 63) / 64;
+  static bool attr_done = false;
+  if (!attr_done) {
+    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<true, ROWMAP, QZERO>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
+    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
+    attr_done = true;
+  }
   for (int i1 = 0; i1 < a.C; i1 += block) {
     const int i2 = (i1 + block < a.C) ? i1 + block : a.C;
     const int nb = i2 - i1;
     if (nb == B)
-      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid), dim3(64), 0, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid), dim3(256), BLOCK_SMEM, st, a, i1, nb);
     else
-      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid), dim3(64), 0, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid), dim3(256), BLOCK_SMEM, st, a, i1, nb);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     if (i2 < a.C) {
