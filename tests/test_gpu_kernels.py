@@ -240,6 +240,27 @@ def test_loop_identity_U_is_round_to_nearest(dev):
     assert torch.equal(Qt.cpu().float(), want)
 
 
+def test_loop_quantizer_arithmetic_is_ieee_exact(dev):
+    """With U = I every column is quantized on its own: 2M (w, s) pairs, including tiny and huge ratios,
+    must give exactly floor(w / s + 8.5) with IEEE division (the kernel hoists a reciprocal out of the chain)."""
+    R, C = 2048, 1024
+    g = torch.Generator().manual_seed(99)
+    W = torch.randn(R, C, generator=g) * 0.02
+    W[:, 100] = 0.0
+    W[:, 101] *= 1e4
+    W[:, 102] *= 1e-6
+    W[5, :] = torch.linspace(-0.2, 0.2, C)
+    s = (torch.rand(C, R, generator=g) * 0.02 + 1e-4).bfloat16().float()
+    s[103] = torch.tensor(1e-12).bfloat16().float()  # the all-zero-group scale
+    s[200:300] = (W.t()[200:300].abs() / 7.5 + 1e-12).bfloat16().float()  # values that land on .5 boundaries often
+    Wt = W.t().contiguous()
+    want = torch.floor(Wt / s + 8.0 + 0.5).clamp(0, 15)
+    Wd = Wt.clone().to(dev)
+    Qt = ops.gptq_loop_(Wd, torch.eye(C, device=dev), s.to(dev), None, None, 8.0, 15.0, torch.bfloat16, 128)
+    assert torch.equal(Qt.cpu().float(), want)
+    assert torch.equal(Wd.cpu(), ((want - 8.0) * s).bfloat16().float())
+
+
 def test_loop_compact_scale_and_perm(dev):
     R, C, g = 128, 512, 64
     W32, U, s, s_rep, z_rep, maxq, perm, perm_inv = _loop_case(R, C, 8, g=g, act_order=True)
