@@ -26,8 +26,10 @@ PEAK_HBM = 8000.0  # GB/s
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=16)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--streams", type=int, default=4,
+                    help="independent linears are queued round-robin on this many HIP streams (1 = one at a time)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
     ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer"],
@@ -145,14 +147,37 @@ def main():
         packed = h.packed_words()
         return h, q, s, packed
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    # Steps are independent linears (each has its own Hessian, factor, codes and words).  One linear is a long
+    # chain of dependent launches that cannot fill the GPU by itself, so consecutive steps go round-robin
+    # onto `streams` HIP streams; nothing in a step reads a value back, the host just queues.
+    main_stream = torch.cuda.current_stream(dev)
+    n_lanes = max(1, args.streams)
+    lanes = [torch.cuda.Stream(device=dev) for _ in range(n_lanes)] if n_lanes > 1 else [main_stream]
+
+    def run(k, lanes):
+        for ln in lanes:
+            if ln is not main_stream:
+                ln.wait_stream(main_stream)
+        last = None
+        t_begin = time.perf_counter()
+        for i in range(k):
+            with torch.cuda.stream(lanes[i % len(lanes)]):
+                last = step()
+        host_ms[0] = (time.perf_counter() - t_begin) * 1e3 / max(k, 1)
+        torch.cuda.synchronize()
+        return last
+
+    host_ms = [0.0]
+    run(args.warmup, lanes)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = step()
-    torch.cuda.synchronize()
+    out = run(args.steps, lanes)
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    host_issue_ms = host_ms[0]
+    # the same step, one at a time on one stream: the latency of a single linear
+    run(1, [main_stream])
+    t0 = time.perf_counter()
+    run(3, [main_stream])
+    ms_single = (time.perf_counter() - t0) * 1e3 / 3
 
     # ---- per-phase device times (HIP events on the stream the kernels run on), outside the timed region
     def timed(fn, reps=3):
@@ -264,8 +289,10 @@ def main():
         "config": {
             "workload": "config 1: expert gate_proj 2048x7168 bf16, 8192 calibration tokens, 4-bit sym g128 B128; "
             "step = Hessian SYRK + factorisation + GPTQ loop + int32 packing",
-            "R": R, "C": C, "tokens": n,
+            "R": R, "C": C, "tokens": n, "streams": n_lanes,
         },
+        "ms_per_step_one_stream": round(ms_single, 3),
+        "host_queueing_ms_per_step": round(host_issue_ms, 3),
         "roofline": roofline,
         "cpu_baseline": cpu,
         "phases": phases,

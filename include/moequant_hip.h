@@ -47,6 +47,33 @@ int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int
  * that a caller accumulating many batches can mirror once at the end). */
 int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
 
+/* ---- (1b) Hessian hygiene before the factorisation ---------------------------------------------------
+ * Device-side restatement of the Hessian part of GPTQ.quantization_pre_step, src/gptq.py:140-146:
+ *   `if torch.isnan(self.H).any().item(): self.H = torch.eye(...)`, `pruned_ids = torch.diag(self.H) == 0`,
+ *   `self.H[pruned_ids, pruned_ids] = 1`.  The reference reads the NaN verdict back to the host; here it
+ *   stays in `flags`, so nothing synchronises.
+ *   upper_only : 1 = H holds only its upper triangle (what mq_hessian_syrk_bf16 leaves with mirror == 0);
+ *                the lower triangle is written here as its mirror image.  0 = H is full, only scanned.
+ *   pruned : out, C bytes, 1 where diag(H) was 0 (the caller treats those weight columns as zero,
+ *            `self.W[:, pruned_ids] = 0`, src/gptq.py:152).
+ *   flags  : out, int32[4]: [0] != 0 when H held a NaN and was replaced by the identity, [1] = number of
+ *            pruned channels; [2] is written by mq_hessian_damp; [3] unused.
+ */
+int mq_hessian_prestep(float* H, long ldh, int C, int upper_only, uint8_t* pruned, int* flags, void* stream);
+
+/* Device-side restatement of the regularisation in GPTQ._get_hessian_inverse, src/gptq.py:221-234:
+ *   `zero_cols = torch.nonzero(w.eq(0).all(dim=0))`, `H[zero_cols, :] = 0`, `H[:, zero_cols] = 0`,
+ *   `H[zero_cols, zero_cols] = 1`, `damp = rel_damp * torch.diag(H).mean()`, `H[diag] += damp`.
+ *   W      : R x C weights (ldw) of type w_dtype, read only; column c counts as zero when every entry is +-0
+ *            or pruned[c] != 0 (pruned nullable).  Column indices of W address rows/columns of H as they are,
+ *            as the reference does (also after an activation-order permutation of H).
+ *   flags  : the array mq_hessian_prestep wrote; [2] receives the number of cleared channels.
+ *   workspace : mq_hessian_damp_workspace_bytes(C) bytes.
+ */
+size_t mq_hessian_damp_workspace_bytes(int C);
+int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_dtype, long ldw, int R, const uint8_t* pruned,
+                    float rel_damp, int* flags, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- (2) damped Cholesky / Cholesky-inverse -------------------------------------------------------
  * In place: A (SPD, upper triangle read, C % 128 == 0) -> unit-diagonal upper-triangular
  * U = chol(A^-1, upper) / diag, strictly lower part zeroed.  Replaces
@@ -56,7 +83,8 @@ int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
  *          from which inv_sym assembles A^-1 = R^-T R^-1.
  *   info : one device int, must be 0 on entry; a non-positive/NaN pivot stores its 1-based index
  *          (the torch path raises LinAlgError there and the caller falls back to identity,
- *          src/gptq.py:239-240).  The output is unspecified when info != 0.
+ *          src/gptq.py:239-240).  When info != 0 the output is the identity matrix: that fallback, taken on
+ *          the device so that the caller need not read info back before queueing the loop.
  */
 int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream);
 

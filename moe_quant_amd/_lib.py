@@ -18,6 +18,9 @@ SIGNATURES = {
     "mq_hessian_syrk_workspace_bytes": (_sz, [_i, _i]),
     "mq_hessian_syrk_bf16": (_i, [_vp, _l, _vp, _l, _i, _i, _f, _f, _i, _vp, _sz, _vp]),
     "mq_symmetrize_upper": (_i, [_vp, _l, _i, _vp]),
+    "mq_hessian_prestep": (_i, [_vp, _l, _i, _i, _vp, _vp, _vp]),
+    "mq_hessian_damp_workspace_bytes": (_sz, [_i]),
+    "mq_hessian_damp": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp, _sz, _vp]),
     "mq_factor_upper_inverse": (_i, [_vp, _l, _i, _i, _vp, _vp]),
     "mq_quant_grid_sym": (_i, [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "mq_prepare_wt": (_i, [_vp, _i, _l, _i, _i, _vp, _vp, _vp, _l, _vp]),

@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libmoequant_hip.so")
-SOURCES = ["gemm_f32.hip", "syrk_bf16.hip", "factor.hip", "gptq_loop.hip", "prep_pack.hip"]
+SOURCES = ["gemm_f32.hip", "syrk_bf16.hip", "factor.hip", "gptq_loop.hip", "prep_pack.hip", "hygiene.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

@@ -237,10 +237,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
 // One workgroup per row.  The diagonal travels through LDS: the one thread that loads it publishes the
 // value before the barrier (a data dependence the compiler cannot reorder), so the thread that later
 // overwrites the diagonal cannot be observed by anyone.
-__global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C, int normalize) {
+// A failed factorisation (*info != 0) leaves the identity, the fallback GPTQ takes when Cholesky raises.
+__global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C, int normalize, const int* info) {
   __shared__ float dsh;
   const int j = blockIdx.x;
   float* row = A + (long)j * ld;
+  if (*info != 0) {
+    for (int k = threadIdx.x; k < C; k += 256) row[k] = (k == j) ? 1.f : 0.f;
+    return;
+  }
   if (threadIdx.x == 0) dsh = row[j];
   __syncthreads();
   const float d = dsh;
@@ -302,6 +307,6 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
     const long p = (long)nfull * 2 * s;
     if (p + s < C && (rc = level(p, (int)(C - p - s), 1)) != MQ_OK) return rc;
   }
-  hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize);
+  hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize, info);
   return mq_check_launch();
 }

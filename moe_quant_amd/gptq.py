@@ -40,7 +40,8 @@ class GPTQ:
     ):
         self._validate_layer(layer)
         self.layer = layer
-        self.W = self.layer.weight
+        self._W = self.layer.weight
+        self._W_lazy = False
         self.d_row, self.d_col = layer.weight.shape[0], int(np.prod(layer.weight.shape[1:]))  # src/model_utils.py:11-12
         self.sym = sym
         self.group_size = group_size
@@ -62,11 +63,59 @@ class GPTQ:
         if tied_gptq_handle is not None:
             tied_gptq_handle.num_tied_handles += 1
         self.issue_zero_samples = False
-        self.issue_nan_hessian = False
-        self.issue_non_invertible = False
+        self._issue_nan_hessian = False
+        self._issue_non_invertible = False
+        # device-side verdicts of the last pre-step / factorisation; read back only when somebody asks
+        self._flags = None
+        self._flags_unread = False
+        self._info = None
+        self._pruned = None
+        self._H_upper_only = False  # H holds only its upper triangle (state of the handle that owns H)
+        self._H_clean = False  # H went through the pre-step scan and nothing touched it since (idem)
         # engine state shared with tied handles (the reference recomputes both for every tied handle)
         self._perm = None
         self._hessian_inv = None
+
+    # The reference keeps three host booleans and pays a device->host read for two of them inside quantize().
+    # Here the verdicts stay on the device (so linears can be queued back to back on several streams) and are
+    # fetched when one of these attributes is read.
+    @property
+    def issue_nan_hessian(self) -> bool:
+        if self._flags_unread and self._flags is not None:
+            self._issue_nan_hessian = self._issue_nan_hessian or bool(self._flags[0].item())
+            self._flags_unread = False
+        return self._issue_nan_hessian
+
+    @issue_nan_hessian.setter
+    def issue_nan_hessian(self, v: bool) -> None:
+        self._issue_nan_hessian, self._flags_unread = bool(v), False
+
+    @property
+    def issue_non_invertible(self) -> bool:
+        if self._info is not None:
+            self._issue_non_invertible = self._issue_non_invertible or int(self._info.item()) != 0
+            self._info = None
+        return self._issue_non_invertible
+
+    @issue_non_invertible.setter
+    def issue_non_invertible(self, v: bool) -> None:
+        self._issue_non_invertible, self._info = bool(v), None
+
+    @property
+    def W(self) -> Tensor:
+        """`layer.weight` before the pre-step; afterwards the fp32 copy with pruned input channels zeroed that
+        the reference keeps (src/gptq.py:148-152), materialised on first use: the kernels read the layer's own
+        weights plus the pruned mask instead."""
+        if self._W_lazy:
+            w = self.layer.weight.detach().clone().float()
+            if self._pruned is not None:
+                w = torch.where(self._pruned.bool()[None, :], torch.zeros((), device=w.device), w)
+            self._W, self._W_lazy = w, False
+        return self._W
+
+    @W.setter
+    def W(self, w: Tensor) -> None:
+        self._W, self._W_lazy = w, False
 
     @staticmethod
     def _validate_layer(layer):
@@ -91,6 +140,7 @@ class GPTQ:
         # only the upper triangle is accumulated; quantization_pre_step mirrors it once
         ops.hessian_syrk_(self.H, input, beta, alpha, mirror=False)
         self._H_upper_only = True
+        self._H_clean = False
         self.num_samples += num_new_samples
 
     add_batch = update
@@ -105,43 +155,58 @@ class GPTQ:
         if self.num_tied_handles == 0:
             self.H = None
             self._hessian_inv = None
+            self._H_upper_only = self._H_clean = False
         elif self.tied_gptq_handle:
             self.tied_gptq_handle.num_tied_handles -= 1
             if self.tied_gptq_handle.num_tied_handles == 0:
                 self.tied_gptq_handle.H = None
                 self.tied_gptq_handle._hessian_inv = None
+                self.tied_gptq_handle._H_upper_only = self.tied_gptq_handle._H_clean = False
         self.num_samples = 0
         self._perm = None
+        self._pruned = None
         if self.tied_gptq_handle is not None:
             self._hessian_inv = None
         torch.cuda.empty_cache()
 
     # ---- pre-step: src/gptq.py:122-154 --------------------------------------------------------------
+    def _hessian_owner(self) -> "GPTQ":
+        t = self.tied_gptq_handle
+        return t if (t is not None and self.H is t.H) else self
+
     def symmetrize_hessian(self) -> None:
         """`update` maintains the upper triangle of H only; this mirrors it onto the lower one."""
-        if self.H is not None and getattr(self, "_H_upper_only", False):
+        owner = self._hessian_owner()
+        if self.H is not None and owner._H_upper_only:
             ops.symmetrize_upper_(self.H)
-            self._H_upper_only = False
+            owner._H_upper_only = False
 
     @torch.no_grad()
     def quantization_pre_step(self) -> None:
-        self.symmetrize_hessian()
         if self.H is None:
             if self.tied_gptq_handle:
                 self.H = self.tied_gptq_handle.H
             else:
                 self.H = torch.eye(self.d_col, device=self.W_device, dtype=torch.float32)
                 self.issue_zero_samples = True
+        if self.H is None:  # tied to a handle that holds no Hessian either
+            self.H = torch.eye(self.d_col, device=self.W_device, dtype=torch.float32)
+            self.issue_zero_samples = True
         if self.is_distributed and torch.distributed.is_available() and torch.distributed.is_initialized():
             if torch.distributed.get_world_size() > 1:
                 raise NotImplementedError("the multi-GPU Hessian all-reduce is outside this engine's scope")
-        if torch.isnan(self.H).any().item():
-            self.H = torch.eye(self.d_col, device=self.W_device, dtype=torch.float32)
-            self.issue_nan_hessian = True
-        pruned_ids = torch.diag(self.H) == 0
-        self.H[pruned_ids, pruned_ids] = 1
-        self.W = self.W.clone().float()
-        self.W[:, pruned_ids] = 0
+        owner = self._hessian_owner()
+        if owner is not self and owner._H_clean:
+            # the owner's pre-step already scanned (and its quantize damped) this very matrix: no NaN, no zero
+            # on the diagonal is left to find (the reference scans it again for every tied handle)
+            self._pruned, self._flags, self._flags_unread = None, None, False
+        else:
+            # NaN -> identity, zero diagonal -> 1 (+ the mirror of the upper triangle), all on the device
+            self._pruned, self._flags = ops.hessian_prestep_(self.H, owner._H_upper_only)
+            self._flags_unread = True
+            owner._H_upper_only = False
+            owner._H_clean = True
+        self._W, self._W_lazy = None, True
         self.pre_step_completed = True
 
     # ---- quantize: src/gptq.py:156-218 ---------------------------------------------------------------
@@ -151,9 +216,9 @@ class GPTQ:
             raise NotImplementedError("only symmetric quantization is supported (as MoE-Quant's README states)")
         d_col, dtype, device = self.d_col, self.W_dtype, self.W_device
         group_size = self.group_size or d_col
-        W = self.W
+        W, dead = self._kernel_weights()
         # per-group scales from the un-updated weights (src/gptq.py:171-178): compact (R,G) and (G,R)
-        scale_rg, scale_gr = ops.quant_grid_sym(W, group_size, bits, dtype)
+        scale_rg, scale_gr = ops.quant_grid_sym(W, group_size, bits, dtype, dead_cols=dead)
         tied = self.tied_gptq_handle
         perm = perm_inv = perm_i32 = perm_inv_i32 = None
         if self.quantization_order == QuantizationOrder.ACTIVATION:
@@ -169,7 +234,7 @@ class GPTQ:
             if tied is None:
                 self.H = self.H[perm][:, perm]
         hessian_inv = self._get_hessian_inverse()
-        Wt = ops.prepare_wt(W, perm_i32)
+        Wt = ops.prepare_wt(W, perm_i32, dead_cols=dead)
         if perm is None:
             scale_row = torch.arange(d_col, device=device, dtype=torch.int32) // group_size
         else:
@@ -182,6 +247,13 @@ class GPTQ:
         scale = scale_rg.to(dtype)
         zero = torch.full_like(scale, qzero)
         return qweight, scale, zero
+
+    def _kernel_weights(self):
+        """(weights, pruned mask) the kernels read: after the pre-step the layer's own weights plus the mask stand
+        for the reference's fp32 copy with zeroed columns, unless somebody has touched or replaced that copy."""
+        if self._W_lazy:
+            return self.layer.weight.detach(), self._pruned
+        return self._W.detach(), None
 
     def quantize(self, bits: int | float) -> Tuple[Tensor, Tensor, Tensor]:
         self.quantization_pre_step()
@@ -198,21 +270,16 @@ class GPTQ:
         tied = self.tied_gptq_handle
         if tied is not None and tied._hessian_inv is not None and tied.H is self.H:
             return tied._hessian_inv  # same damped H -> same factor; the reference recomputes it
-        w = self.W
-        zero_cols = torch.nonzero(w.eq(0).all(dim=0))
         H = self.H
         if not tied:
-            H[zero_cols, :] = 0
-            H[:, zero_cols] = 0
-            H[zero_cols, zero_cols] = 1
-            damp = self.rel_damp * torch.diag(self.H).mean()
-            self.H.diagonal().add_(damp)
-        U, info = linalg_utils.inverse_cholesky_factor(H)
-        if int(info.item()) != 0:
-            # the reference's bare `except` around cholesky lands here (src/gptq.py:239-240); it never sets
-            # issue_non_invertible, this engine does
-            self.issue_non_invertible = True
-            U = torch.eye(self.d_col, device=H.device, dtype=torch.float32)
+            # all-zero weight columns -> unit rows/columns of H, then damping (src/gptq.py:221-234)
+            flags = self._flags if self._flags is not None else torch.zeros(4, dtype=torch.int32, device=H.device)
+            w, pruned = self._kernel_weights()
+            ops.hessian_damp_(H, w, pruned, self.rel_damp, flags)
+            self._H_clean = True
+        # a failed factorisation yields the identity on the device, the reference's `except` branch
+        # (src/gptq.py:239-240, which never sets issue_non_invertible; this engine does)
+        U, self._info = linalg_utils.inverse_cholesky_factor(H)
         if self.num_tied_handles > 0:
             self._hessian_inv = U
         return U

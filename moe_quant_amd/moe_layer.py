@@ -60,8 +60,14 @@ def quantize_moe_layer(
     keep_outputs: bool = False,
     keep_codes: Optional[List[int]] = None,
     max_rows_per_update: int = 1 << 17,
+    streams: int = 4,
 ) -> LayerResult:
-    """x (T, C) bf16 on the GPU, expert_ids (T, top_k) int64 on the GPU."""
+    """x (T, C) bf16 on the GPU, expert_ids (T, top_k) int64 on the GPU.
+
+    `streams`: experts are quantized round-robin on that many HIP streams.  One linear is a long chain of
+    dependent launches whose tail (small trailing updates behind one-workgroup diagonal blocks) leaves most
+    of the GPU idle; independent linears on other streams fill it.  Nothing in the per-linear path reads a
+    value back to the host, so one host thread keeps all streams fed."""
     dev = x.device
     E = len(experts)
     keep_codes = set(keep_codes or [])
@@ -100,34 +106,50 @@ def quantize_moe_layer(
     sync()
     res.seconds["hessians_incl_gather_and_forward"] = time.perf_counter() - t1
 
-    # ---- phase 2: quantize + pack 3 linears per expert
+    # ---- phase 2: quantize + pack 3 linears per expert, experts round-robin over the streams
     t2 = time.perf_counter()
-    issues = {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
+    main = torch.cuda.current_stream(dev)
+    lanes = [torch.cuda.Stream(device=dev) for _ in range(max(1, streams))] if streams > 1 else [main]
+    for s_ in lanes:
+        if s_ is not main:
+            s_.wait_stream(main)
+    done = []  # handles whose verdict words are read after everything is queued
     for e, (g, u, d) in enumerate(handles):
-        if e in keep_codes:
-            g.symmetrize_hessian()
-            d.symmetrize_hessian()
-            if g.H is not None:
-                res.hessians[f"{e}.gate_proj"] = g.H.clone()
-            if d.H is not None:
-                res.hessians[f"{e}.down_proj"] = d.H.clone()
-        for name, h in (("gate_proj", g), ("up_proj", u), ("down_proj", d)):
-            q, s, z = h.quantize(bits)
-            words = h.packed_words()
-            issues["zero_samples"] += int(h.issue_zero_samples)
-            issues["nan_hessian"] += int(h.issue_nan_hessian)
-            issues["non_invertible"] += int(h.issue_non_invertible)
-            if keep_outputs:
-                res.packed[f"{e}.{name}"] = words
-                res.scales[f"{e}.{name}"] = s
+        lane = lanes[e % len(lanes)]
+        with torch.cuda.stream(lane):
             if e in keep_codes:
-                res.qweight[f"{e}.{name}"] = q
-                res.scales[f"{e}.{name}"] = s
-        for h in (g, u, d):  # as quant.py:330: free per-linear state as soon as the linear is done
-            h.H = None
-            h._hessian_inv = None
-            h.W = h.layer.weight
+                g.symmetrize_hessian()
+                d.symmetrize_hessian()
+                if g.H is not None:
+                    res.hessians[f"{e}.gate_proj"] = g.H.clone()
+                if d.H is not None:
+                    res.hessians[f"{e}.down_proj"] = d.H.clone()
+            for name, h in (("gate_proj", g), ("up_proj", u), ("down_proj", d)):
+                q, s, z = h.quantize(bits)
+                words = h.packed_words()
+                done.append(h)
+                if keep_outputs:
+                    res.packed[f"{e}.{name}"] = words
+                    res.scales[f"{e}.{name}"] = s
+                if e in keep_codes:
+                    res.qweight[f"{e}.{name}"] = q
+                    res.scales[f"{e}.{name}"] = s
+            for h in (g, u, d):  # as quant.py:330: free per-linear state as soon as the linear is done
+                if h.H is not None and lane is not main:
+                    h.H.record_stream(lane)  # allocated on the main stream, last used on this one
+                h.H = None
+                h._hessian_inv = None
+                h._Qt = None
+                h.W = h.layer.weight
+    for s_ in lanes:
+        if s_ is not main:
+            main.wait_stream(s_)
     sync()
+    issues = {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
+    for h in done:
+        issues["zero_samples"] += int(h.issue_zero_samples)
+        issues["nan_hessian"] += int(h.issue_nan_hessian)
+        issues["non_invertible"] += int(h.issue_non_invertible)
     res.seconds["quantize_and_pack"] = time.perf_counter() - t2
     res.seconds["total"] = time.perf_counter() - t0
     res.issues = issues

@@ -36,13 +36,14 @@ def _p(t: Optional[Tensor]) -> Optional[int]:
 
 
 class _Workspace:
-    """One growing scratch buffer per device so the hot path does not hit the allocator."""
+    """One growing scratch buffer per (device, stream, purpose), so the hot path does not hit the allocator and
+    linears queued on different streams never share scratch memory."""
 
     def __init__(self):
         self.buf = {}
 
-    def get(self, device: torch.device, nbytes: int) -> Tensor:
-        key = (device.type, device.index)
+    def get(self, device: torch.device, nbytes: int, purpose: str = "") -> Tensor:
+        key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream, purpose)
         b = self.buf.get(key)
         if b is None or b.numel() < nbytes:
             b = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -67,7 +68,7 @@ def hessian_syrk_(H: Tensor, X: Tensor, beta: float, alpha: float, mirror: bool 
         X = X.contiguous()
     n = X.shape[0]
     need = lib.mq_hessian_syrk_workspace_bytes(n, C)
-    ws = _ws.get(H.device, need) if need else None
+    ws = _ws.get(H.device, need, "syrk") if need else None
     ldx = X.stride(0) if n > 1 else C
     rc = lib.mq_hessian_syrk_bf16(
         H.data_ptr(), H.stride(0), X.data_ptr() if n else None, ldx, n, C, beta, alpha, int(mirror),
@@ -85,6 +86,42 @@ def symmetrize_upper_(H: Tensor) -> Tensor:
     if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
         raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
     check(lib.mq_symmetrize_upper(H.data_ptr(), H.stride(0), C, _stream(H)), "mq_symmetrize_upper")
+    return H
+
+
+def hessian_prestep_(H: Tensor, upper_only: bool) -> Tuple[Tensor, Tensor]:
+    """In place: mirror the upper triangle (when `upper_only`), NaN -> identity, zero diagonal entries -> 1.
+    Returns (pruned (C,) uint8, flags (4,) int32), both on the device; nothing is read back."""
+    _dev(H)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    pruned = torch.empty(C, dtype=torch.uint8, device=H.device)
+    flags = torch.empty(4, dtype=torch.int32, device=H.device)
+    rc = lib.mq_hessian_prestep(H.data_ptr(), H.stride(0), C, int(upper_only), pruned.data_ptr(), flags.data_ptr(),
+                                _stream(H))
+    check(rc, "mq_hessian_prestep")
+    return pruned, flags
+
+
+def hessian_damp_(H: Tensor, W: Tensor, pruned: Optional[Tensor], rel_damp: float, flags: Tensor) -> Tensor:
+    """In place: rows/columns of H for all-zero (or pruned) weight columns cleared with a unit diagonal, then
+    rel_damp * mean(diag) added to the diagonal."""
+    _dev(H, W, pruned, flags)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    if W.dim() != 2 or W.shape[1] != C:
+        raise ValueError("W must be (R,C)")
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    need = lib.mq_hessian_damp_workspace_bytes(C)
+    ws = _ws.get(H.device, need, "damp")
+    rc = lib.mq_hessian_damp(H.data_ptr(), H.stride(0), C, W.data_ptr(), _dt(W.dtype), W.stride(0), W.shape[0],
+                             _p(pruned), float(rel_damp), flags.data_ptr(), ws.data_ptr(), need, _stream(H))
+    check(rc, "mq_hessian_damp")
     return H
 
 
@@ -150,7 +187,7 @@ def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor]
     if scale_row is None and scale.shape[0] != C:
         raise ValueError("scale must be (C,R) when no scale_row map is given")
     Qt = torch.empty(C, R, dtype=torch.uint8, device=Wt.device)
-    E = _ws.get(Wt.device, 128 * R * 4)
+    E = _ws.get(Wt.device, 128 * R * 4, "loop")
     rc = lib.mq_gptq_loop(Wt.data_ptr(), Wt.stride(0), C, R, U.data_ptr(), U.stride(0), scale.data_ptr(),
                           scale.stride(0), _p(scale_row), _p(qzero), qzero_const, maxq, _dt(round_dtype), block,
                           Qt.data_ptr(), E.data_ptr(), _stream(Wt))

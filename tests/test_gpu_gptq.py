@@ -149,6 +149,32 @@ def test_tied_handles_share_hessian_and_factor(dev):
     up.reset()
 
 
+def test_streams_give_the_same_bits(dev):
+    """Linears queued on several streams (no host synchronisation between them) equal the one-at-a-time results."""
+    cases = [(synth.weight(128, 512, 30 + i), synth.activations_outlier(700, 512, 40 + i)) for i in range(6)]
+
+    def one(W, X):
+        h = GPTQ(_layer(W, dev), 128, True)
+        h.update(X)
+        q, s, _ = h.quantize(4)
+        return q, s, h.packed_words(), h
+
+    Xs = [X.to(dev) for _, X in cases]
+    serial = [one(W, X) for (W, _), X in zip(cases, Xs)]
+    torch.cuda.synchronize()
+    lanes = [torch.cuda.Stream(device=dev) for _ in range(3)]
+    for ln in lanes:
+        ln.wait_stream(torch.cuda.current_stream(dev))
+    par = []
+    for i, ((W, _), X) in enumerate(zip(cases, Xs)):
+        with torch.cuda.stream(lanes[i % 3]):
+            par.append(one(W, X))
+    torch.cuda.synchronize()
+    for a, b in zip(serial, par):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+        assert not b[3].has_hessian_issues()
+
+
 # ---------------------------------------------------------------- module-level drop-ins
 def test_gptq_loop_and_grid_functions(dev):
     R, C, g = 96, 384, 128

@@ -147,10 +147,94 @@ def test_factor_reports_non_pd(dev):
     A = H.to(dev)
     info = ops.factor_upper_inverse_(A)
     assert int(info.item()) == 201
+    assert torch.equal(A.cpu(), torch.eye(C))  # the fallback GPTQ takes when Cholesky raises, src/gptq.py:239-240
     H = _spd(C, 78)
     H[5, 9] = float("nan")
     info = ops.factor_upper_inverse_(H.to(dev))
     assert int(info.item()) != 0
+
+
+# ---------------------------------------------------------------- Hessian hygiene (src/gptq.py:140-146, 221-234)
+def _prestep_reference(H):
+    """The torch statements of quantization_pre_step on a full matrix."""
+    H = H.clone()
+    nan = bool(torch.isnan(H).any())
+    if nan:
+        H = torch.eye(H.shape[0])
+    pruned = torch.diag(H) == 0
+    H[pruned, pruned] = 1
+    return H, pruned, nan
+
+
+@pytest.mark.parametrize("C", [64, 200, 448])
+@pytest.mark.parametrize("upper_only", [True, False])
+def test_hessian_prestep(dev, C, upper_only):
+    _say(f"prestep C={C} upper_only={upper_only}")
+    X = _rand((3 * C, C), 11 + C)
+    X[:, [5, C - 1]] = 0  # two input channels that never fire
+    H = X.t() @ X / X.shape[0]
+    H = torch.triu(H) + torch.triu(H, 1).t()  # exactly symmetric
+    ref, pruned_ref, _ = _prestep_reference(H)
+    Hd = (torch.triu(H) + torch.tril(torch.full_like(H, 7.0), -1)) if upper_only else H.clone()
+    Hd = Hd.to(dev)
+    pruned, flags = ops.hessian_prestep_(Hd, upper_only)
+    assert torch.equal(Hd.cpu(), ref)
+    assert torch.equal(pruned.cpu().bool(), pruned_ref)
+    assert flags.cpu().tolist()[:2] == [0, 2]
+
+
+@pytest.mark.parametrize("where", ["upper", "diag", "lower"])
+def test_hessian_prestep_nan_gives_identity(dev, where):
+    C = 192
+    H = _spd(C, 3)
+    r, c = {"upper": (10, 150), "diag": (70, 70), "lower": (150, 10)}[where]
+    H[r, c] = float("nan")
+    Hd = H.to(dev)
+    pruned, flags = ops.hessian_prestep_(Hd, False)
+    assert flags[0].item() != 0 and flags[1].item() == 0
+    assert torch.equal(Hd.cpu(), torch.eye(C)) and not pruned.any().item()
+    if where != "lower":  # with upper_only the lower triangle is never read
+        Hd = H.to(dev)
+        pruned, flags = ops.hessian_prestep_(Hd, True)
+        assert flags[0].item() != 0 and torch.equal(Hd.cpu(), torch.eye(C))
+
+
+@pytest.mark.parametrize("R,C,dtype", [(96, 256, torch.bfloat16), (50, 200, torch.bfloat16), (33, 130, torch.float32),
+                                       (64, 136, torch.float16)])
+def test_hessian_damp(dev, R, C, dtype):
+    _say(f"damp R={R} C={C} {dtype}")
+    H = _spd(C, 21 + C)
+    W = _rand((R, C), 5, 0.02).to(dtype)
+    W[:, [3, C - 2]] = 0
+    W[0, 3] = -0.0
+    pruned = torch.zeros(C, dtype=torch.uint8)
+    pruned[[9, 40]] = 1
+    # torch statements of _get_hessian_inverse on the weights with pruned columns zeroed
+    w = W.float().clone()
+    w[:, pruned.bool()] = 0
+    ref = H.clone()
+    zero_cols = torch.nonzero(w.eq(0).all(dim=0))
+    ref[zero_cols, :] = 0
+    ref[:, zero_cols] = 0
+    ref[zero_cols, zero_cols] = 1
+    damp = 0.01 * torch.diag(ref).mean()
+    ref[range(C), range(C)] += damp
+    Hd = H.to(dev)
+    flags = torch.zeros(4, dtype=torch.int32, device=dev)
+    ops.hessian_damp_(Hd, W.to(dev), pruned.to(dev), 0.01, flags)
+    out = Hd.cpu()
+    assert flags[2].item() == 4
+    off = ~torch.eye(C, dtype=torch.bool)
+    assert torch.equal(out[off], ref[off])
+    # the mean runs in another order than torch's: the damping term may differ in its last bits
+    assert torch.allclose(out.diag(), ref.diag(), rtol=1e-6, atol=0)
+    # no dead channel: only the diagonal moves
+    Hd = H.to(dev)
+    ops.hessian_damp_(Hd, torch.ones(R, C, dtype=dtype, device=dev), None, 0.05, flags)
+    assert flags[2].item() == 0
+    ref2 = H.clone()
+    ref2[range(C), range(C)] += 0.05 * torch.diag(H).mean()
+    assert torch.equal(Hd.cpu()[off], H[off]) and torch.allclose(Hd.cpu().diag(), ref2.diag(), rtol=1e-6, atol=0)
 
 
 def test_inv_sym(dev):
