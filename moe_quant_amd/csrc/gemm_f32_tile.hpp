@@ -5,9 +5,16 @@
 
 namespace gemmf32 {
 
-constexpr int BM = 128, BN = 128, BK = 32, LDT = 132;  // LDT: padded LDS row length (floats)
-constexpr int STAGE = BK * LDT;                        // floats per operand per stage
-constexpr size_t SMEM_BYTES = (size_t)4 * STAGE * sizeof(float);  // 2 stages x {A, B}
+constexpr int BM = 128, BN = 128, BK = 32;
+// LDS staging layouts, chosen by how the operand lies in memory so that global float4 loads go to LDS as
+// float4 stores, untransposed:
+//   k-contiguous operand : [x][LDK]  (x = m or n), LDK = BK + 4; a lane fetches its 4 k-values with one b128 read
+//   x-contiguous operand : [k][LDT],  LDT = 128 + 4;              a lane fetches them with four b32 reads
+// A 32x32x2 MFMA sums two k-slots (lanes 0-31 and 32-63).  Which two k meet in one instruction is free as
+// long as A and B agree: per group of 8 k, lane half h owns k = 4h..4h+3 and instruction t pairs (t, 4+t).
+constexpr int LDK = BK + 4, LDT = BM + 4;
+constexpr int STAGE = (BM * LDK > BK * LDT) ? BM * LDK : BK * LDT;  // floats per operand per stage
+constexpr size_t SMEM_BYTES = (size_t)4 * STAGE * sizeof(float);    // 2 stages x {A, B}
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id; give every XCD one contiguous
 // run of tiles so that tiles sharing operand panels meet in the same L2.
@@ -31,6 +38,19 @@ struct TileLoader {
   // Loads a (128 x BK) operand tile: element (x, k) at p[x*sx + k*sk], x in [x0, x0+128), k in [k0, k0+BK).
   static constexpr int NV = BM * BK / 4 / 256;  // float4 per thread
   float4 r[NV];
+  // interior tile: every element exists and every row is 16-byte aligned -> straight-line float4 loads
+  __device__ __forceinline__ void load_fast(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = tid + it * 256;
+      const float* q;
+      if (KCONTIG) q = p + (long)(x0 + idx / (BK / 4)) * sx + k0 + ((idx % (BK / 4)) << 2);
+      else q = p + (long)(k0 + (idx >> 5)) * sk + x0 + ((idx & 31) << 2);
+      // through the native vector type: a struct copy straight from memory left the loader in scratch
+      const floatx4 v = *reinterpret_cast<const floatx4*>(q);
+      r[it] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  }
   __device__ __forceinline__ void load(const float* __restrict__ p, long sx, long sk, int x0, int X, int k0, int Kend,
                                        bool vec_ok, int tid) {
 #pragma unroll
@@ -80,10 +100,7 @@ struct TileLoader {
       const int idx = tid + it * 256;
       if (KCONTIG) {
         const int x = idx / (BK / 4), k = (idx % (BK / 4)) << 2;
-        s[(k + 0) * LDT + x] = r[it].x;
-        s[(k + 1) * LDT + x] = r[it].y;
-        s[(k + 2) * LDT + x] = r[it].z;
-        s[(k + 3) * LDT + x] = r[it].w;
+        *reinterpret_cast<float4*>(&s[x * LDK + k]) = r[it];
       } else {
         const int k = idx >> 5, x = (idx & 31) << 2;
         *reinterpret_cast<float4*>(&s[k * LDT + x]) = r[it];
@@ -100,20 +117,23 @@ struct TileLoader {
 struct NoSink {
   __device__ __forceinline__ void operator()(int, int, float) const {}
 };
-template <bool A_KC, bool B_KC, bool LDS_OUT = false, typename Sink = NoSink>
-__device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int z, float* smem, int vecA, int vecB,
-                                          Sink sink = Sink()) {
+
+// the four k-values (k = 8j + 4h + t, t = 0..3) of operand row x for this lane
+template <bool KC>
+__device__ __forceinline__ float4 frag4(const float* __restrict__ s, int x, int j, int h) {
+  if (KC) return *reinterpret_cast<const float4*>(&s[x * LDK + 8 * j + 4 * h]);
+  const float* q = s + (8 * j + 4 * h) * LDT + x;
+  return make_float4(q[0], q[LDT], q[2 * LDT], q[3 * LDT]);
+}
+
+template <bool A_KC, bool B_KC, bool FAST, bool LDS_OUT, typename Sink>
+__device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int kb, int ke, const float* __restrict__ A,
+                                          const float* __restrict__ B, float* C, float* smem, int vecA, int vecB,
+                                          Sink& sink) {
   float* As = smem;
   float* Bs = smem + 2 * STAGE;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const float* __restrict__ A = g.A + (long)z * g.batchA;
-  const float* __restrict__ B = g.B + (long)z * g.batchB;
-  float* C = g.C + (long)z * g.batchC;
-  const int m0 = tm * BM, n0 = tn * BN;
-  int kb = 0, ke = g.K;
-  if (g.ktrim == 1) ke = min(g.K, m0 + BM);
-  if (g.ktrim == 2) kb = m0;
   const int lr = lane & 31, lk = lane >> 5;
   const float alpha = g.alpha, beta = g.beta;
 
@@ -130,11 +150,19 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
 
   TileLoader<A_KC> la;
   TileLoader<B_KC> lb;
+// (a macro, not a lambda: loaders captured by reference end up in scratch memory)
+#define MQ_GEMM_FETCH(k0)                                       \
+  do {                                                          \
+    if (FAST) {                                                 \
+      la.load_fast(A, g.sam, g.sak, m0, (k0), tid);             \
+      lb.load_fast(B, g.sbn, g.sbk, n0, (k0), tid);             \
+    } else {                                                    \
+      la.load(A, g.sam, g.sak, m0, g.M, (k0), ke, vecA, tid);   \
+      lb.load(B, g.sbn, g.sbk, n0, g.N, (k0), ke, vecB, tid);   \
+    }                                                           \
+  } while (0)
   const int nk = (ke - kb + BK - 1) / BK;
-  if (nk > 0) {
-    la.load(A, g.sam, g.sak, m0, g.M, kb, ke, vecA, tid);
-    lb.load(B, g.sbn, g.sbk, n0, g.N, kb, ke, vecB, tid);
-  }
+  if (nk > 0) MQ_GEMM_FETCH(kb);
   if (beta != 0.f) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -144,7 +172,7 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-          if (row < g.M && col < g.N) cold[i][j][v] = C[(long)row * g.ldc + col];
+          if (FAST || (row < g.M && col < g.N)) cold[i][j][v] = C[(long)row * g.ldc + col];
         }
       }
   }
@@ -155,21 +183,22 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      la.load(A, g.sam, g.sak, m0, g.M, kb + (kt + 1) * BK, ke, vecA, tid);
-      lb.load(B, g.sbn, g.sbk, n0, g.N, kb + (kt + 1) * BK, ke, vecB, tid);
-    }
-    const float* as = As + cur * STAGE + wm * 64 + lr;
-    const float* bs = Bs + cur * STAGE + wn * 64 + lr;
+    if (kt + 1 < nk) MQ_GEMM_FETCH(kb + (kt + 1) * BK);
+    const float* as = As + cur * STAGE;
+    const float* bs = Bs + cur * STAGE;
 #pragma unroll
-    for (int kp = 0; kp < BK / 2; ++kp) {
-      const int k = 2 * kp + lk;
-      const float a0 = as[k * LDT], a1 = as[k * LDT + 32];
-      const float b0 = bs[k * LDT], b1 = bs[k * LDT + 32];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    for (int j = 0; j < BK / 8; ++j) {
+      const float4 a0 = frag4<A_KC>(as, wm * 64 + lr, j, lk), a1 = frag4<A_KC>(as, wm * 64 + 32 + lr, j, lk);
+      const float4 b0 = frag4<B_KC>(bs, wn * 64 + lr, j, lk), b1 = frag4<B_KC>(bs, wn * 64 + 32 + lr, j, lk);
+      const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
+      const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[t], bv0[t], acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[t], bv1[t], acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[t], bv0[t], acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[t], bv1[t], acc[1][1], 0, 0, 0);
+      }
     }
     if (kt + 1 < nk) {
       la.store(As + (cur ^ 1) * STAGE, tid);
@@ -186,7 +215,7 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-        if (row < g.M && col < g.N) {
+        if (FAST || (row < g.M && col < g.N)) {
           float r = alpha * acc[i][j][v];
           if (beta != 0.f) r = fmaf(beta, cold[i][j][v], r);
           if (LDS_OUT) sink(row - m0, col - n0, r);
@@ -194,6 +223,30 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
         }
       }
     }
+#undef MQ_GEMM_FETCH
+}
+
+// One 128x128 output tile (tm, tn) of problem g (batch index z).  smem: SMEM_BYTES of LDS.
+// The old C tile is fetched before the K loop (when beta != 0) so its latency hides behind the products;
+// it is added after the accumulation, never fed through the accumulator.
+// Interior tiles (whole tile inside the matrix, aligned rows, K range a multiple of BK) run a copy of the
+// body without any bounds test: guarded loads sit in branches, and a branch makes the wavefront wait for
+// every load in flight.
+// With LDS_OUT the result tile is not written to memory: it is handed to `sink(r, c, value)` (tile-local
+// coordinates) after the last LDS operand read, so the sink may overwrite the staging buffers.
+template <bool A_KC, bool B_KC, bool LDS_OUT = false, typename Sink = NoSink>
+__device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int z, float* smem, int vecA, int vecB,
+                                          Sink sink = Sink()) {
+  const float* __restrict__ A = g.A + (long)z * g.batchA;
+  const float* __restrict__ B = g.B + (long)z * g.batchB;
+  float* C = g.C + (long)z * g.batchC;
+  const int m0 = tm * BM, n0 = tn * BN;
+  int kb = 0, ke = g.K;
+  if (g.ktrim == 1) ke = min(g.K, m0 + BM);
+  if (g.ktrim == 2) kb = m0;
+  const bool interior = vecA && vecB && m0 + BM <= g.M && n0 + BN <= g.N && ((ke - kb) % BK == 0);
+  if (interior) tile_core<A_KC, B_KC, true, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
+  else tile_core<A_KC, B_KC, false, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
 }
 
 __device__ __forceinline__ void decode_tile(const GemmF32& g, int L, int tiles_n, int& tm, int& tn) {
