@@ -9,6 +9,8 @@
 // eight coalesced 4-byte loads, transposes it in registers and writes two 16-byte rows into an LDS
 // tile laid out [channel][token].  With too few tiles to fill 256 CUs the token range is split; the
 // partial tiles go to a caller-provided workspace and are reduced in a fixed order (deterministic).
+#include <cstdlib>
+
 #include "common.hpp"
 
 extern "C" int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
@@ -399,6 +401,179 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 }
 
+// =============================================================================================
+// Same 256x256 workgroup tile, staged without touching the vector registers: the token-major rows of X go
+// from memory straight into LDS (16 bytes per lane per instruction) and the matrix-core operands, which want
+// the tokens of one channel side by side, are read back with the transposing LDS load.
+//
+// LDS stage = 32 tokens x 512 channels (the 256 of the row tile, then the 256 of the column tile) cut into
+// 1 KB chunks [token quad q][channel group G of 128]; a chunk is what one wavefront-wide direct load writes
+// (lane i fills bytes 16i..16i+15).  Inside a chunk, eight blocks of 128 bytes hold 4 tokens x 16 channels
+// each, token-major: lane i of the load fetches token (i%8)/2, channels 16*(i/8) + 8*(i%2) ... +7.
+// A transposing read (ds_read_b64_tr_b16) has the 16 lanes of a group fetch 8 bytes each from one such block
+// -- 128 contiguous bytes, no bank conflict -- and hands lane s the 4 tokens of channel s.  Two of them give a
+// lane its 8 tokens of a 32x32x16 operand; which tokens share a lane is irrelevant as long as both operands
+// use the same rule, and both are read by the same code.
+// Four stages are allocated: while stage s feeds the matrix cores, stages s+1..s+3 are in flight, tracked
+// with the vector-memory counter (8 loads per wavefront per stage), one barrier per stage.
+// =============================================================================================
+constexpr int KT3 = 32, NST3 = 4, CHUNK3 = 1024;
+constexpr int STAGE3 = (KT3 / 4) * 4 * CHUNK3;  // bytes
+constexpr size_t DMA_SMEM = (size_t)NST3 * STAGE3;
+
+typedef __attribute__((address_space(3))) void* lds_void_p;
+typedef __attribute__((address_space(1))) const void* gbl_void_p;
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+// One wavefront-wide direct load: lane i copies 16 bytes from its own global address to LDS byte lds_addr + 16 i.
+// Written as inline assembly on purpose: told about an LDS-writing load, the compiler drains all of them
+// (vmcnt(0)) before the next LDS read, which would serialise the stages this kernel keeps in flight.  The
+// kernel orders loads and reads itself (s_waitcnt vmcnt + barrier below).
+__device__ __forceinline__ void dma16(const void* gptr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
+// issues (or, for ragged stages, completes) the 8 chunk loads of this wavefront for the stage starting at token t0.
+// wave_u is the wavefront index as a scalar; lane_ptr = X + tau*ldx + 16*b + 8*half for this lane's slot.
+template <bool FAST>
+__device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, const uint16_t* lane_ptr, long ldx, int t0, int tend,
+                                          int C, int m0, int n0, unsigned char* buf, unsigned lds_base, int wave_u,
+                                          int lane) {
+  const int b = lane >> 3, tau = (lane & 7) >> 1, half = lane & 1;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int ch = wave_u * 8 + i, q = ch >> 2, G = ch & 3;
+    const int chan0 = ((G & 2) ? n0 : m0) + (G & 1) * 128;  // scalar
+    if (FAST) {
+      const long off = (long)(t0 + 4 * q) * ldx + chan0;  // scalar
+      dma16(lane_ptr + off, lds_base + (unsigned)(ch * CHUNK3));
+    } else {
+      const int chan = chan0 + 16 * b + 8 * half;
+      const int tok = t0 + 4 * q + tau;
+      const bool ok = (tok < tend) && (chan + 8 <= C);
+      const uint16_t* src = X + (long)(tok < tend ? tok : tend - 1) * ldx + (chan + 8 <= C ? chan : 0);
+      uint4 v = *reinterpret_cast<const uint4*>(src);
+      if (!ok) v = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4*>(buf + ch * CHUNK3 + lane * 16) = v;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_kernel(
+    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
+    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: LDS targets of the direct loads live in M0
+  const int wm = wave >> 1, wn = wave & 1;
+  const int L = xcd_remap(blockIdx.x, ntri * splits);
+  const int split = L / ntri;
+  int tm, tn;
+  blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
+  const int m0 = tm * T2, n0 = tn * T2;
+  const int tbeg = split * tokens_per_split;
+  const int tend = min(n, tbeg + tokens_per_split);
+  const int nk = (tend - tbeg + KT3 - 1) / KT3;
+  const bool interior = (m0 + T2 <= C) && (n0 + T2 <= C);
+  // LDS byte address of the staging area plus this wavefront's share of a stage, as a scalar
+  const unsigned smem_lds = __builtin_amdgcn_readfirstlane(
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem);
+  const uint16_t* lane_ptr = X + (long)((lane & 7) >> 1) * ldx + 16 * (lane >> 3) + 8 * (lane & 1);
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+#define MQ_SYRK_ISSUE(st)                                                                         \
+  do {                                                                                            \
+    const int t0_ = tbeg + (st)*KT3;                                                              \
+    unsigned char* buf_ = smem + ((st) % NST3) * STAGE3;                                          \
+    const unsigned lds_ = smem_lds + (unsigned)(((st) % NST3) * STAGE3);                          \
+    if (interior && t0_ + KT3 <= tend) dma_stage<true>(X, lane_ptr, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);  \
+    else dma_stage<false>(X, lane_ptr, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);        \
+  } while (0)
+
+#pragma unroll
+  for (int st = 0; st < NST3 - 1; ++st)
+    if (st < nk) MQ_SYRK_ISSUE(st);
+
+  // fragment addressing: 16-lane group g16 = lane/16 -> channel block parity g16&1, token half g16>>1
+  const int g16 = lane >> 4, s16 = lane & 15;
+  const int a_off = wm * CHUNK3 + (g16 & 1) * 128 + s16 * 8;        // + i*256 (block pair i) + quad*4*CHUNK3
+  const int b_off = (2 + wn) * CHUNK3 + (g16 & 1) * 128 + s16 * 8;  // + j*256
+  const int hq = g16 >> 1;
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // stage kt must have landed: at most the loads of the stages issued after it may still be in flight
+    const int ahead = min(nk, kt + NST3 - 1) - (kt + 1);
+    // (lgkmcnt(0) as well: LDS writes of a ragged stage must have landed before the barrier lets others read)
+    asm volatile("" ::: "memory");
+    if (ahead >= 2) __builtin_amdgcn_s_waitcnt(0x4070);       // vmcnt(16) lgkmcnt(0)
+    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);                  // vmcnt(0) lgkmcnt(0)
+    // a bare barrier: __syncthreads() carries a fence that makes the compiler drain every direct load in flight.
+    // The empty asm statements keep the compiler from moving LDS accesses across it.
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + NST3 - 1 < nk) MQ_SYRK_ISSUE(kt + NST3 - 1);
+    const unsigned char* stg = smem + (kt % NST3) * STAGE3;
+#pragma unroll
+    for (int kk = 0; kk < KT3 / 16; ++kk) {
+      short4v fa[4][2], fb[4][2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int quad = 4 * kk + 2 * r + hq;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          fa[i][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(stg + quad * 4 * CHUNK3 + a_off + i * 256));
+          fb[i][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(stg + quad * 4 * CHUNK3 + b_off + i * 256));
+        }
+      }
+      bf16x8 va[4], vb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        va[i] = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        vb[i] = __builtin_shufflevector(fb[i][0], fb[i][1], 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8n, va[i]),
+                                                              __builtin_bit_cast(bf16x8n, vb[j]), acc[i][j], 0, 0, 0);
+    }
+  }
+#undef MQ_SYRK_ISSUE
+
+  const int lr = lane & 31, lk = lane >> 5;
+  const bool partial = splits > 1;
+  float* out = partial ? ws + ((long)split * ntri + (L - split * ntri)) * (T2 * T2) : H;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = wn * 128 + j * 32 + lr;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+        if (partial) {
+          out[r * T2 + c] = acc[i][j][v];
+        } else if (m0 + r < C && n0 + c < C) {
+          float* q = H + (long)(m0 + r) * ldh + n0 + c;
+          float val = alpha * acc[i][j][v];
+          if (beta != 0.f) val = fmaf(beta, *q, val);
+          *q = val;
+        }
+      }
+    }
+}
+
 // fixed-order sum of the split partials of the big kernel; upper tiles only
 __global__ __launch_bounds__(256) void syrk_big_reduce_kernel(float* __restrict__ H, long ldh, int C, float alpha,
                                                               float beta, int ntri, int splits,
@@ -525,13 +700,21 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
       if (!workspace || workspace_bytes < need) return MQ_ERR_WORKSPACE;
     }
     static bool big_attr = false;
+    static bool use_dma = true;
     if (!big_attr) {
       (void)hipFuncSetAttribute((const void*)syrk_bf16_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)BIG_SMEM);
+      (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)DMA_SMEM);
+      use_dma = getenv("MQ_SYRK_OLD") == nullptr;
       big_attr = true;
     }
-    hipLaunchKernelGGL(syrk_bf16_big_kernel, dim3(ntri * splits), dim3(256), BIG_SMEM, st, H, ldh, (const uint16_t*)X,
-                       ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    if (use_dma)
+      hipLaunchKernelGGL(syrk_bf16_dma_kernel, dim3(ntri * splits), dim3(256), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
+                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    else
+      hipLaunchKernelGGL(syrk_bf16_big_kernel, dim3(ntri * splits), dim3(256), BIG_SMEM, st, H, ldh, (const uint16_t*)X,
+                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     if (splits > 1) {
