@@ -429,14 +429,17 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 // Written as inline assembly on purpose: told about an LDS-writing load, the compiler drains all of them
 // (vmcnt(0)) before the next LDS read, which would serialise the stages this kernel keeps in flight.  The
 // kernel orders loads and reads itself (s_waitcnt vmcnt + barrier below).
-__device__ __forceinline__ void dma16(const void* gptr, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory", "m0");
+// The address is a scalar base plus a 32-bit per-lane byte offset, so a stage costs scalar arithmetic only.
+__device__ __forceinline__ void dma16(const void* sbase, unsigned lane_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sbase), "s"(lds_addr)
+               : "memory", "m0");
 }
 
 // issues (or, for ragged stages, completes) the 8 chunk loads of this wavefront for the stage starting at token t0.
-// wave_u is the wavefront index as a scalar; lane_ptr = X + tau*ldx + 16*b + 8*half for this lane's slot.
+// wave_u is the wavefront index as a scalar; lane_off = 2*(tau*ldx + 16*b + 8*half), the byte offset of this
+// lane's slot inside a chunk's source (4 token rows x 128 channels).
 template <bool FAST>
-__device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, const uint16_t* lane_ptr, long ldx, int t0, int tend,
+__device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsigned lane_off, long ldx, int t0, int tend,
                                           int C, int m0, int n0, unsigned char* buf, unsigned lds_base, int wave_u,
                                           int lane) {
   const int b = lane >> 3, tau = (lane & 7) >> 1, half = lane & 1;
@@ -446,7 +449,7 @@ __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, const 
     const int chan0 = ((G & 2) ? n0 : m0) + (G & 1) * 128;  // scalar
     if (FAST) {
       const long off = (long)(t0 + 4 * q) * ldx + chan0;  // scalar
-      dma16(lane_ptr + off, lds_base + (unsigned)(ch * CHUNK3));
+      dma16(X + off, lane_off, lds_base + (unsigned)(ch * CHUNK3));
     } else {
       const int chan = chan0 + 16 * b + 8 * half;
       const int tok = t0 + 4 * q + tau;
@@ -470,15 +473,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int split = L / ntri;
   int tm, tn;
   blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
+  // uniform values that the division and the square root above left in vector registers: back to scalars,
+  // the direct loads take their base address and LDS target from scalar registers
+  tm = __builtin_amdgcn_readfirstlane(tm);
+  tn = __builtin_amdgcn_readfirstlane(tn);
   const int m0 = tm * T2, n0 = tn * T2;
-  const int tbeg = split * tokens_per_split;
+  const int tbeg = __builtin_amdgcn_readfirstlane(split * tokens_per_split);
   const int tend = min(n, tbeg + tokens_per_split);
   const int nk = (tend - tbeg + KT3 - 1) / KT3;
   const bool interior = (m0 + T2 <= C) && (n0 + T2 <= C);
   // LDS byte address of the staging area plus this wavefront's share of a stage, as a scalar
   const unsigned smem_lds = __builtin_amdgcn_readfirstlane(
       (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem);
-  const uint16_t* lane_ptr = X + (long)((lane & 7) >> 1) * ldx + 16 * (lane >> 3) + 8 * (lane & 1);
+  const unsigned lane_off = 2u * (unsigned)(((lane & 7) >> 1) * ldx + 16 * (lane >> 3) + 8 * (lane & 1));
 
   floatx16 acc[4][4];
 #pragma unroll
@@ -493,8 +500,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int t0_ = tbeg + (st)*KT3;                                                              \
     unsigned char* buf_ = smem + ((st) % NST3) * STAGE3;                                          \
     const unsigned lds_ = smem_lds + (unsigned)(((st) % NST3) * STAGE3);                          \
-    if (interior && t0_ + KT3 <= tend) dma_stage<true>(X, lane_ptr, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);  \
-    else dma_stage<false>(X, lane_ptr, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);        \
+    if (interior && t0_ + KT3 <= tend) dma_stage<true>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);  \
+    else dma_stage<false>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);        \
   } while (0)
 
 #pragma unroll
