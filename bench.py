@@ -152,7 +152,7 @@ def main():
     # onto `streams` HIP streams; nothing in a step reads a value back, the host just queues.
     main_stream = torch.cuda.current_stream(dev)
     n_lanes = max(1, args.streams)
-    lanes = [torch.cuda.Stream(device=dev) for _ in range(n_lanes)] if n_lanes > 1 else [main_stream]
+    lanes = [main_stream] + [torch.cuda.Stream(device=dev) for _ in range(n_lanes - 1)]  # the current stream is lane 0
 
     def run(k, lanes):
         for ln in lanes:

@@ -109,7 +109,7 @@ def quantize_moe_layer(
     # ---- phase 2: quantize + pack 3 linears per expert, experts round-robin over the streams
     t2 = time.perf_counter()
     main = torch.cuda.current_stream(dev)
-    lanes = [torch.cuda.Stream(device=dev) for _ in range(max(1, streams))] if streams > 1 else [main]
+    lanes = [main] + [torch.cuda.Stream(device=dev) for _ in range(max(1, streams) - 1)]  # the current stream is lane 0
     for s_ in lanes:
         if s_ is not main:
             s_.wait_stream(main)
