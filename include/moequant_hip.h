@@ -43,6 +43,17 @@ size_t mq_hessian_syrk_workspace_bytes(int n, int C);
 int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
                          int mirror, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same accumulation for `groups` independent Hessians of one width C in one call (the experts of an MoE
+ * block: the reference loops over forward hooks, one addmm_ per expert, src/gptq.py:97-103 via quant.py:258-277).
+ * H, ldh, X, ldx, n, beta, alpha are HOST arrays with one entry per problem; the device pointers they hold follow
+ * the rules above.  When every problem has n >= 256 tokens and 16-byte aligned rows, up to 16 problems share a
+ * launch and no workspace is touched; otherwise each problem runs as a plain mq_hessian_syrk_bf16 call with the
+ * given workspace (mq_hessian_syrk_grouped_workspace_bytes = the largest single requirement). */
+size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C);
+int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, const void* const* X, const long* ldx,
+                                 const int* n, int C, const float* beta, const float* alpha, int mirror, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
 /* lower triangle <- transpose of the upper triangle (what mirror != 0 does after the accumulation; exported so
  * that a caller accumulating many batches can mirror once at the end). */
 int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);

@@ -462,14 +462,15 @@ __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsign
   }
 }
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_kernel(
-    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
-    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+// one 256x256 tile (or one token split of it); bid = linear workgroup index among ntri*splits
+__device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx,
+                                              int n, int C, float alpha, float beta, int ntri, int splits,
+                                              int tokens_per_split, float* __restrict__ ws, int bid,
+                                              unsigned char* smem) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: LDS targets of the direct loads live in M0
   const int wm = wave >> 1, wn = wave & 1;
-  const int L = xcd_remap(blockIdx.x, ntri * splits);
+  const int L = xcd_remap(bid, ntri * splits);
   const int split = L / ntri;
   int tm, tn;
   blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
@@ -579,6 +580,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
       }
     }
+}
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_kernel(
+    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
+    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  syrk_dma_tile(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+}
+
+// Several independent accumulations (one Hessian each, same C) in one launch: blockIdx.y picks the problem.
+// Each workgroup runs the whole token range of its tile, so no partial tiles and no workspace: the groups,
+// not token splits, supply the parallelism (C = 2048 has only 36 tiles per problem).
+constexpr int SYRK_MAX_GROUP = 16;
+struct SyrkGroupTable {
+  float* H[SYRK_MAX_GROUP];
+  const uint16_t* X[SYRK_MAX_GROUP];
+  long ldh[SYRK_MAX_GROUP], ldx[SYRK_MAX_GROUP];
+  int n[SYRK_MAX_GROUP];
+  float alpha[SYRK_MAX_GROUP], beta[SYRK_MAX_GROUP];
+};
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_grouped_kernel(
+    SyrkGroupTable t, int C, int ntri) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int z = blockIdx.y;
+  const int tps = (t.n[z] + KT3 - 1) / KT3 * KT3;
+  syrk_dma_tile(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
+                smem);
 }
 
 // fixed-order sum of the split partials of the big kernel; upper tiles only
@@ -752,4 +780,63 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
     rc = mq_check_launch();
   }
   return rc;
+}
+
+// Host arrays of `groups` entries each.  Problems that the direct-load kernel cannot take (few tokens, unaligned
+// rows) make the whole call fall back to one plain call per problem, so the result never depends on the path.
+extern "C" size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C) {
+  size_t need = 0;
+  for (int g = 0; g < groups; ++g) {
+    const size_t w = mq_hessian_syrk_workspace_bytes(n[g], C);
+    if (w > need) need = w;
+  }
+  return need;
+}
+
+extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, const void* const* X,
+                                            const long* ldx, const int* n, int C, const float* beta, const float* alpha,
+                                            int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+  if (groups < 0 || C <= 0 || (groups > 0 && (!H || !ldh || !X || !ldx || !n || !beta || !alpha))) return MQ_ERR_ARG;
+  bool fast = groups > 1;
+  for (int g = 0; g < groups; ++g) {
+    if (!H[g] || n[g] < 0 || ldh[g] < C || (n[g] > 0 && (!X[g] || ldx[g] < C))) return MQ_ERR_ARG;
+    if (n[g] <= 0 || !use_big(X[g], ldx[g], n[g], C)) fast = false;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (!fast) {
+    for (int g = 0; g < groups; ++g) {
+      const int rc = mq_hessian_syrk_bf16(H[g], ldh[g], X[g], ldx[g], n[g], C, beta[g], alpha[g], mirror, workspace,
+                                          workspace_bytes, stream);
+      if (rc != MQ_OK) return rc;
+    }
+    return MQ_OK;
+  }
+  static bool attr_done = false;
+  if (!attr_done) {
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_grouped_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)DMA_SMEM);
+    attr_done = true;
+  }
+  const int tiles = (C + T2 - 1) / T2, ntri = tiles * (tiles + 1) / 2;
+  for (int g0 = 0; g0 < groups; g0 += SYRK_MAX_GROUP) {
+    const int cnt = groups - g0 < SYRK_MAX_GROUP ? groups - g0 : SYRK_MAX_GROUP;
+    SyrkGroupTable t;
+    for (int i = 0; i < SYRK_MAX_GROUP; ++i) {
+      const int g = g0 + (i < cnt ? i : 0);
+      t.H[i] = H[g];
+      t.X[i] = (const uint16_t*)X[g];
+      t.ldh[i] = ldh[g];
+      t.ldx[i] = ldx[g];
+      t.n[i] = n[g];
+      t.alpha[i] = alpha[g];
+      t.beta[i] = beta[g];
+    }
+    hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel, dim3(ntri, cnt), dim3(256), DMA_SMEM, st, t, C, ntri);
+    int rc = mq_check_launch();
+    if (rc != MQ_OK) return rc;
+    if (mirror)
+      for (int i = 0; i < cnt; ++i)
+        if ((rc = mq_symmetrize_upper(H[g0 + i], ldh[g0 + i], C, stream)) != MQ_OK) return rc;
+  }
+  return MQ_OK;
 }

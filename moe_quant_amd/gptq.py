@@ -145,6 +145,29 @@ class GPTQ:
 
     add_batch = update
 
+    @staticmethod
+    @torch.no_grad()
+    def update_many(handles, inputs) -> None:
+        """`h.update(x)` for several handles of one input width with one library call (the experts of a block,
+        whose hooks the reference serves one addmm_ at a time).  Same arithmetic per handle as `update`."""
+        Hs, Xs, betas, alphas = [], [], [], []
+        for h, x in zip(handles, inputs):
+            x = x.reshape(-1, x.shape[-1])
+            if x.dtype != torch.bfloat16:
+                raise TypeError(f"GPTQ.update needs bf16 activations, got {x.dtype}")
+            if x.shape[0] == 0:
+                continue
+            if h.H is None:
+                h.H = torch.zeros((h.d_col, h.d_col), device=x.device, dtype=torch.float32)
+            n = x.shape[0]
+            Hs.append(h.H)
+            Xs.append(x)
+            betas.append(h.num_samples / (h.num_samples + n))
+            alphas.append(2.0 / (h.num_samples + n))
+            h.num_samples += n
+            h._H_upper_only, h._H_clean = True, False
+        ops.hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror=False)
+
     @property
     def tokens_collected(self) -> int:
         return self.num_samples

@@ -78,6 +78,37 @@ def hessian_syrk_(H: Tensor, X: Tensor, beta: float, alpha: float, mirror: bool 
     return H
 
 
+def hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror: bool = True) -> None:
+    """H_i <- beta_i*H_i + alpha_i*X_i^T X_i for several Hessians of one width in one call (lists of equal length)."""
+    import ctypes as C_
+
+    lib = _lib.load()
+    k = len(Hs)
+    if not (len(Xs) == len(betas) == len(alphas) == k):
+        raise ValueError("Hs, Xs, betas, alphas must have the same length")
+    if k == 0:
+        return
+    _dev(*Hs, *Xs)
+    C = Hs[0].shape[0]
+    Xs = [x if (x.shape[0] == 0 or x.stride(1) == 1) else x.contiguous() for x in Xs]
+    for H, X in zip(Hs, Xs):
+        if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+            raise ValueError("every H must be a (C,C) fp32 matrix with unit column stride")
+        if X.dtype != torch.bfloat16 or X.dim() != 2 or X.shape[1] != C:
+            raise ValueError("every X must be (n,C) bf16")
+    ns = (C_.c_int * k)(*[x.shape[0] for x in Xs])
+    Hp = (C_.c_void_p * k)(*[h.data_ptr() for h in Hs])
+    Xp = (C_.c_void_p * k)(*[(x.data_ptr() if x.shape[0] else None) for x in Xs])
+    ldh = (C_.c_long * k)(*[h.stride(0) for h in Hs])
+    ldx = (C_.c_long * k)(*[(x.stride(0) if x.shape[0] > 1 else C) for x in Xs])
+    be = (C_.c_float * k)(*[float(b) for b in betas])
+    al = (C_.c_float * k)(*[float(a) for a in alphas])
+    need = lib.mq_hessian_syrk_grouped_workspace_bytes(k, ns, C)
+    ws = _ws.get(Hs[0].device, need, "syrk") if need else None
+    rc = lib.mq_hessian_syrk_bf16_grouped(k, Hp, ldh, Xp, ldx, ns, C, be, al, int(mirror), _p(ws), need, _stream(Hs[0]))
+    check(rc, "mq_hessian_syrk_bf16_grouped")
+
+
 def symmetrize_upper_(H: Tensor) -> Tensor:
     """Copies the upper triangle of H onto the lower one, in place."""
     _dev(H)

@@ -149,6 +149,25 @@ def test_tied_handles_share_hessian_and_factor(dev):
     up.reset()
 
 
+def test_update_many_equals_update(dev):
+    Ws = [synth.weight(64, 512, 60 + i) for i in range(3)]
+    Xa = [synth.activations_outlier(400 + 100 * i, 512, 70 + i).to(dev) for i in range(3)]
+    Xb = [synth.activations_outlier(300, 512, 80 + i).to(dev) for i in range(3)]
+    one = [GPTQ(_layer(W, dev), 128, True) for W in Ws]
+    many = [GPTQ(_layer(W, dev), 128, True) for W in Ws]
+    for h, a, b in zip(one, Xa, Xb):
+        h.update(a)
+        h.update(b)
+    GPTQ.update_many(many, Xa)
+    GPTQ.update_many(many, Xb)
+    for h1, h2 in zip(one, many):
+        assert h1.num_samples == h2.num_samples
+        q1, s1, _ = h1.quantize(4)
+        q2, s2, _ = h2.quantize(4)
+        assert (h1.H - h2.H).norm() / h1.H.norm() < 1e-6
+        assert (q1 == q2).float().mean().item() >= 0.999 and torch.equal(s1, s2)
+
+
 def test_streams_give_the_same_bits(dev):
     """Linears queued on several streams (no host synchronisation between them) equal the one-at-a-time results."""
     cases = [(synth.weight(128, 512, 30 + i), synth.activations_outlier(700, 512, 40 + i)) for i in range(6)]

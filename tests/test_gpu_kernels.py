@@ -95,6 +95,28 @@ def test_hessian_running_mean_matches_oracle(dev):
     assert ((H.cpu() - Href).norm() / Href.norm()).item() < 1e-5
 
 
+@pytest.mark.parametrize("C,ns", [(512, [700, 300, 1500, 256, 4000]), (256, [300] * 18), (384, [100, 600, 0])])
+def test_hessian_syrk_grouped(dev, C, ns):
+    """Several Hessians in one call: each within the 1e-5 gate of fp64 and equal to the one-at-a-time result up to
+    the order of the fp32 token sum."""
+    _say(f"grouped syrk C={C} ns={ns}")
+    Xs = [synth.activations_outlier(n, C, seed=50 + i) for i, n in enumerate(ns)]
+    H0 = [_rand((C, C), 70 + i) for i in range(len(ns))]
+    H0 = [h + h.t() for h in H0]
+    betas = [0.25 * (i % 3) for i in range(len(ns))]
+    alphas = [2.0 / max(n, 1) for n in ns]
+    Hg = [h.clone().to(dev) for h in H0]
+    ops.hessian_syrk_grouped_(Hg, [x.to(dev) for x in Xs], betas, alphas, mirror=True)
+    for i, n in enumerate(ns):
+        ref = betas[i] * H0[i].double() + alphas[i] * (Xs[i].double().t() @ Xs[i].double())
+        got = Hg[i].cpu().double()
+        assert ((got - ref).norm() / ref.norm()).item() < 1e-5, (i, n)
+        assert torch.equal(got, got.t())
+        Hs = H0[i].clone().to(dev)
+        ops.hessian_syrk_(Hs, Xs[i].to(dev), betas[i], alphas[i])
+        assert ((Hs.cpu().double() - got).norm() / ref.norm()).item() < 1e-6
+
+
 def test_hessian_upper_only(dev):
     C, n = 512, 512
     X = synth.activations_outlier(n, C, seed=3).to(dev)
