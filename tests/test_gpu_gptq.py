@@ -83,6 +83,82 @@ def test_config1_full_size(dev):
     _run_case(synth.config1(1.0), dev, chunks=1)
 
 
+def test_config2_full_size(dev):
+    """Config 2 at its real shape: 7168x2048 down projection, 65536 SwiGLU tokens, packing included."""
+    _run_case(synth.config2(1.0), dev, chunks=4)
+
+
+def _full_size_properties(dev, R, C, n, g, act_order, seed):
+    """Shapes the CPU oracle cannot finish in seconds: checks that do not depend on size.  Inputs are drawn on
+    the GPU.  (1) Hessian against torch's fp32 product; (2) U H U^T is diagonal for the factor the loop gets;
+    (3) scales equal the oracle's closed form; codes in range; packed words unpack to the codes; (4) rows are
+    independent: quantizing the first 256 rows alone gives the same codes bit for bit; (5) the GPTQ codes beat
+    round-to-nearest on the layer-output error tr(dH d^T)."""
+    from moe_quant_amd import linalg_utils
+
+    _say(f"full-size properties R={R} C={C} n={n} g={g} act_order={act_order}")
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    W = (torch.randn(R, C, generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    order = "activation" if act_order else "default"
+    h = GPTQ(_layer(W, dev), g, True, 0.01, 128, quantization_order=order)
+    Href = torch.zeros(C, C, device=dev)
+    outl = synth.outlier_channels(C, seed + 1).to(dev)
+    step = 16384
+    for s0 in range(0, n, step):
+        x = torch.randn(min(step, n - s0), C, generator=gen, device=dev)
+        x[:, outl] *= 20.0
+        x = x.to(torch.bfloat16)
+        h.update(x)
+        Href.addmm_(x.float().t(), x.float())
+        del x
+    Href.mul_(2.0 / n)
+    h.symmetrize_hessian()
+    assert ((h.H - Href).norm() / Href.norm()).item() < 1e-5
+    H0 = h.H.clone()  # undamped, unpermuted
+    q, s, z = h.quantize(4)
+    assert not h.has_hessian_issues()
+    # (2) the factor of the damped (and permuted) Hessian the handle now holds
+    U, info = linalg_utils.inverse_cholesky_factor(h.H)
+    assert int(info.item()) == 0
+    T = U @ h.H @ U.t()
+    d = T.diagonal().clone()
+    T.diagonal().zero_()
+    assert (T.norm() / d.norm()).item() < 1e-3
+    del T, U
+    # (3)
+    sc_ref = O.find_quantization_meta(W.cpu().float().reshape(R, C // g, g), 4, torch.bfloat16)[0]
+    assert torch.equal(s.cpu().float(), sc_ref.reshape(R, C // g).float())
+    assert q.dtype == torch.uint8 and int(q.max()) <= 15
+    words = h.packed_words()
+    assert torch.equal(O.unpack_from_int32(words.cpu(), 4, (R, C)), q.cpu().to(torch.int8) - 8)
+    # (4)
+    h2 = GPTQ(_layer(W[:256].contiguous(), dev), g, True, 0.01, 128, quantization_order=order)
+    h2.H, h2.num_samples = H0.clone(), n
+    q2, _, _ = h2.quantize(4)
+    assert torch.equal(q2, q[:256])
+    # (5) on a row sample, in fp32 on the GPU
+    Wd = W[:512].float()
+    Wq = dequantize_linear_weight(q[:512], s[:512], z[:512]).float()
+    sg = s[:512].float().repeat_interleave(g, dim=1)
+    rtn = (torch.clamp(torch.floor(Wd / sg + 8.5), 0, 15) - 8) * sg
+    e_gptq = get_relative_mse_error(Wq, Wd, H0).item()
+    e_rtn = get_relative_mse_error(rtn, Wd, H0).item()
+    _say(f"  rel-mse gptq {e_gptq:.4e}  round-to-nearest {e_rtn:.4e}")
+    assert e_gptq < e_rtn
+
+
+def test_config4_o_proj_full_size_properties(dev):
+    _full_size_properties(dev, 7168, 16384, 16384, 128, False, 4400)
+
+
+def test_config5_gate_up_full_size_properties(dev):
+    _full_size_properties(dev, 18432, 7168, 65536, 64, True, 5500)
+
+
+def test_config5_down_full_size_properties(dev):
+    _full_size_properties(dev, 7168, 18432, 65536, 128, True, 5510)
+
+
 # ---------------------------------------------------------------- fallbacks of the reference (src/gptq.py:129-152,224-240)
 def test_zero_samples_is_round_to_nearest(dev):
     W = synth.weight(128, 256, 1)
