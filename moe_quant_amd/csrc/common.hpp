@@ -49,6 +49,10 @@ struct GemmF32 {
   int tri, ktrim;
   int batch;
   long batchA, batchB, batchC;
+  // optional: the B operand is the sum of several arrays of the same layout, bsum_stride elements apart;
+  // column tile tn adds the first min(bsum, tn / bsum_c + 1) of them (0 = plain B).  Interior tiles only.
+  int bsum, bsum_c;
+  long bsum_stride;
 };
 int mq_launch_gemm_f32(const GemmF32& g, hipStream_t stream);
 bool mq_gemm_operand_aligned(const float* p, long ld, long batch);

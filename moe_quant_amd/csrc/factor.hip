@@ -11,10 +11,16 @@
 //     diag kernel  : R_bb = revchol(H_bb), then R_bb^-1 written in place (one workgroup, LDS resident)
 //     panel GEMM   : R_ab = H_ab * (R_bb^-1)^T            for a < b   (fp32 MFMA)
 //     trailing GEMM: H_aa' -= R_ab R_a'b^T                for a <= a' < b  (fp32 MFMA, upper tiles only)
-//   triangular inverse, block size s = 128, 256, ...: for each aligned pair (left, right)
-//     T^T = U22^T R12^T  (written to the unused mirror position below the diagonal)
-//     U12 = -U11 T
+//   triangular inverse, one block row at a time, bottom to top, riding along in the same launches:
+//     row b:  T^T = U22^T R12^T   (U22 = finished inverse of everything below/right of b, R12 = R[b, b+1:];
+//                                  written to the unused mirror position below the diagonal)
+//             U[b, b+1:] = -U_bb T
+//     Both products only touch rows >= b, the elimination at step b only rows < b, so the first runs as extra
+//     workgroups of step b's trailing-update launch and the second as extra workgroups of step b-1's panel
+//     launch: the (1/3)C^3 flop of the inverse fill the CUs the late elimination steps leave idle.
 //   finalize: U[j, k] /= U[j, j], strictly lower part zeroed.
+#include <cstdlib>
+
 #include "gemm_f32_tile.hpp"
 
 namespace {
@@ -22,6 +28,7 @@ namespace {
 constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
 constexpr int LDM = 131;   // LDS row pitch (odd: lane-per-row accesses hit 32 distinct banks)
+static int INV_KC = 4;  // the first inverse product is cut into K chunks of 4 blocks (512), one workgroup each
 
 // ---------------------------------------------------------------------------------------------
 // Diagonal block: S (128x128, upper valid) -> R^-1 where S = R R^T, R upper.
@@ -204,17 +211,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void r
   diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false);
 }
 
+// Work item idx of the first inverse product: (row tile tm, K chunk s), enumerated from the bottom row tile up.
+// Chunk s of row tile tm is written 128*s columns to the right of chunk 0; the second product adds the chunks
+// while it loads its B operand (a fixed order, and no fence or atomic between workgroups: a device-scope fence
+// here writes back the L2 of the XCD, dirty with the trailing update, and cost more than it saved).
+__device__ __forceinline__ void inv_first_tile(const GemmF32& ginv, int kc, int idx, float* buf) {
+  using namespace gemmf32;
+  const int T = ginv.M / NB, smax = (T + kc - 1) / kc;
+  const int tm = T - 1 - idx / smax, s = idx % smax;
+  if (s > tm / kc) return;  // U22 is triangular: row tile tm stops at k = (tm+1)*128
+  const int k0 = s * kc * NB, k1 = min((s + 1) * kc * NB, (tm + 1) * NB);
+  GemmF32 gl = ginv;
+  gl.A += (long)k0 * gl.sak;
+  gl.B += (long)k0 * gl.sbk;
+  gl.C += s * NB;
+  gl.K = k1 - k0;
+  gl.ktrim = 0;
+  tile_body<false, true>(gl, tm, 0, 0, buf, 1, 1);
+}
+
+__global__ __launch_bounds__(256) void inv_first_kernel(GemmF32 ginv, int kc) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  inv_first_tile(ginv, kc, blockIdx.x, reinterpret_cast<float*>(smem));
+}
+
 // One launch per elimination step b (block at offset i1, panel P = A[0:i1, i1:i1+128] already solved):
-//   workgroup 0        : updates the next diagonal tile (rows/cols [i1-128, i1)) with the panel, keeps the
-//                        result in LDS and inverts it right away (the next step's critical path);
-//   workgroups 1..T-1  : the other T-1 upper tiles of the trailing update  A[0:i1,0:i1] -= P P^T.
-// The diagonal-block work is thereby hidden behind the bulk of the trailing update.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void trail_diag_kernel(GemmF32 g, int total, float* A,
+//   workgroup 0          : updates the next diagonal tile (rows/cols [i1-128, i1)) with the panel, keeps the
+//                          result in LDS and inverts it right away (the next step's critical path);
+//   next inv_tiles ones  : T^T = U22^T R12^T for block row b of the inverse: row tile tm (k <= its last row, U22 is
+//                          triangular) times K chunk s of 512; chunk s lands 128*s columns to the right of chunk
+//                          0, in the mirror area of block column b+s, free since that row's inverse is complete;
+//                          the second product sums the chunks while loading them;
+//   the rest             : the other T-1 upper tiles of the trailing update  A[0:i1,0:i1] -= P P^T.
+// The diagonal-block work is thereby hidden behind the bulk of the trailing update, and the inverse behind both.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void trail_diag_kernel(GemmF32 g, int total, GemmF32 ginv,
+                                                                                                  int inv_tiles, int kc, float* A,
                                                                                                   long ld, int i1, int* info) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* buf = reinterpret_cast<float*>(smem);
   using namespace gemmf32;
-  if (blockIdx.x == 0) {
+  const int bid = blockIdx.x;
+  if (bid == 0) {
     const int t = i1 / NB - 1;  // last tile of the column-major upper-triangle order
     tile_body<true, true, true>(g, t, t, 0, buf, 1, 1, [&](int r, int c, float v) {
       if (c >= r) Sv(buf, r, c) = v;
@@ -225,13 +262,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
     }
     __syncthreads();
     diag_block_invert(buf, A + (long)(i1 - NB) * ld + (i1 - NB), ld, i1 - NB, info, true);
+  } else if (bid <= inv_tiles) {
+    inv_first_tile(ginv, kc, bid - 1, buf);
   } else {
     int tm, tn;
-    tri_decode(xcd_remap(blockIdx.x - 1, total - 1), tm, tn);
+    tri_decode(xcd_remap(bid - 1 - inv_tiles, total - 1), tm, tn);
     tile_body<true, true>(g, tm, tn, 0, buf, 1, 1);
   }
 }
 
+// Panel product of step b (P = H_ab Dinv^T, one tile per row block) together with the second product of the
+// inverse's block row b+1 (U12 = -U11 T, one tile per column block): two independent GEMMs in one launch.
+__global__ __launch_bounds__(256) void panel_inv_kernel(GemmF32 gp, int panel_tiles, GemmF32 g2, int inv_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* buf = reinterpret_cast<float*>(smem);
+  using namespace gemmf32;
+  const int bid = blockIdx.x;
+  if (bid < panel_tiles) tile_body<true, true>(gp, bid, 0, 0, buf, 1, 1);
+  else tile_body<true, true>(g2, 0, bid - panel_tiles, 0, buf, 1, 1);
+}
 
 // U[j,k] <- U[j,k] / U[j,j] for k > j, 1 on the diagonal, 0 for k < j (normalize == 0: only the zeroing).
 // One workgroup per row.  The diagonal travels through LDS: the one thread that loads it publishes the
@@ -267,45 +316,69 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
   hipStream_t st = (hipStream_t)stream;
   static bool attr_done = false;
   if (!attr_done) {
+    if (const char* e = getenv("MQ_INV_KC")) INV_KC = atoi(e) > 0 ? atoi(e) : INV_KC;
     (void)hipFuncSetAttribute((const void*)revchol_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)DIAG_SMEM);
     (void)hipFuncSetAttribute((const void*)trail_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)FUSED_SMEM);
+    (void)hipFuncSetAttribute((const void*)panel_inv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)gemmf32::SMEM_BYTES);
+    (void)hipFuncSetAttribute((const void*)inv_first_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)gemmf32::SMEM_BYTES);
     attr_done = true;
   }
   if ((ld & 3) || ((uintptr_t)A & 15)) return MQ_ERR_ARG;  // float4 access to rows of A
   int rc;
+  // the two products of block row b of the inverse (w = columns to the right of b)
+  auto inv_first = [&](int b, int& tiles) {  // T^T (w x 128) = U22^T (w x w) * R12^T (w x 128), in K chunks
+    const long p = (long)b * NB;
+    const int w = C - (int)p - NB;
+    tiles = (w / NB) * ((w / NB + INV_KC - 1) / INV_KC);
+    return GemmF32{A + (p + NB) * ld + (p + NB), A + p * ld + (p + NB), A + (p + NB) * ld + p, 1, ld, 1, ld, ld,
+                   w, NB, w, 1.f, 0.f, 0, 1, 1, 0, 0, 0};
+  };
+  auto inv_second = [&](int b, int& tiles) {  // U12 (128 x w) = -U11 (128 x 128) * T,  T(k,n) = Tt[n][k]
+    const long p = (long)b * NB;
+    const int w = C - (int)p - NB;
+    tiles = w / NB;
+    return GemmF32{A + p * ld + p, A + (p + NB) * ld + p, A + p * ld + (p + NB), ld, 1, 1, ld, ld,
+                   NB, w, NB, -1.f, 0.f, 0, 0, 1, 0, 0, 0, (w / NB + INV_KC - 1) / INV_KC, INV_KC, NB};
+  };
+  const int B = C / NB;
   hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, A, ld, C - NB, info);
   if ((rc = mq_check_launch()) != MQ_OK) return rc;
-  for (int i1 = C - NB; i1 > 0; i1 -= NB) {
+  for (int b = B - 1; b >= 1; --b) {
+    const int i1 = b * NB;
     float* P = A + i1;  // panel: rows [0,i1), cols [i1, i1+NB)
     const float* Dinv = A + (long)i1 * ld + i1;
     GemmF32 panel{P, Dinv, P, ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
-    if ((rc = mq_launch_gemm_f32(panel, st)) != MQ_OK) return rc;
+    int t2 = 0;
+    GemmF32 g2 = panel;
+    if (b + 1 <= B - 2) g2 = inv_second(b + 1, t2);  // row b+1: its T was produced in the previous launch
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(b + t2), dim3(256), gemmf32::SMEM_BYTES, st, panel, b, g2, t2);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     const int tiles = i1 / NB, total = tiles * (tiles + 1) / 2;
-    hipLaunchKernelGGL(trail_diag_kernel, dim3(total), dim3(256), FUSED_SMEM, st, trail, total, A, ld, i1, info);
+    int t1 = 0;
+    GemmF32 g1 = trail;
+    if (b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
+    hipLaunchKernelGGL(trail_diag_kernel, dim3(total + t1), dim3(256), FUSED_SMEM, st, trail, total, g1, t1, INV_KC, A, ld,
+                       i1, info);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
-  for (long s = NB; s < C; s *= 2) {
-    const int nfull = (int)(C / (2 * s));
-    auto level = [&](long p, int w, int batch) -> int {
-      float* U11 = A + p * ld + p;
-      float* U22 = A + (p + s) * ld + (p + s);
-      float* R12 = A + p * ld + (p + s);
-      float* Tt = A + (p + s) * ld + p;
-      const long bs = 2 * s * (ld + 1);
-      // T^T (w x s) = U22^T (w x w) * R12^T (w x s)
-      GemmF32 g1{U22, R12, Tt, 1, ld, 1, ld, ld, w, (int)s, w, 1.f, 0.f, 0, 1, batch, bs, bs, bs};
-      int r = mq_launch_gemm_f32(g1, st);
-      if (r != MQ_OK) return r;
-      // U12 (s x w) = -U11 (s x s) * T (s x w),  T(k,n) = Tt[n][k]
-      GemmF32 g2{U11, Tt, R12, ld, 1, 1, ld, ld, (int)s, w, (int)s, -1.f, 0.f, 0, 2, batch, bs, bs, bs};
-      return mq_launch_gemm_f32(g2, st);
-    };
-    if (nfull > 0 && (rc = level(0, (int)s, nfull)) != MQ_OK) return rc;
-    const long p = (long)nfull * 2 * s;
-    if (p + s < C && (rc = level(p, (int)(C - p - s), 1)) != MQ_OK) return rc;
+  // what is left of the inverse once the elimination has reached the top: second product of row 1, both of row 0
+  if (B >= 3) {
+    int t2;
+    GemmF32 g2 = inv_second(1, t2);
+    if ((rc = mq_launch_gemm_f32(g2, st)) != MQ_OK) return rc;
+  }
+  if (B >= 2) {
+    int t;
+    GemmF32 g1 = inv_first(0, t);
+    hipLaunchKernelGGL(inv_first_kernel, dim3(t), dim3(256), gemmf32::SMEM_BYTES, st, g1, INV_KC);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
+    GemmF32 g2 = inv_second(0, t);
+    if ((rc = mq_launch_gemm_f32(g2, st)) != MQ_OK) return rc;
   }
   hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize, info);
   return mq_check_launch();

@@ -51,6 +51,21 @@ struct TileLoader {
       r[it] = make_float4(v[0], v[1], v[2], v[3]);
     }
   }
+  // r += the same tile of another array
+  __device__ __forceinline__ void add_fast(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = tid + it * 256;
+      const float* q;
+      if (KCONTIG) q = p + (long)(x0 + idx / (BK / 4)) * sx + k0 + ((idx % (BK / 4)) << 2);
+      else q = p + (long)(k0 + (idx >> 5)) * sk + x0 + ((idx & 31) << 2);
+      const floatx4 v = *reinterpret_cast<const floatx4*>(q);
+      r[it].x += v[0];
+      r[it].y += v[1];
+      r[it].z += v[2];
+      r[it].w += v[3];
+    }
+  }
   __device__ __forceinline__ void load(const float* __restrict__ p, long sx, long sk, int x0, int X, int k0, int Kend,
                                        bool vec_ok, int tid) {
 #pragma unroll
@@ -150,12 +165,14 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
 
   TileLoader<A_KC> la;
   TileLoader<B_KC> lb;
+  const int nsum = g.bsum ? min(g.bsum, (n0 / BN) / g.bsum_c + 1) : 1;  // arrays summed into the B operand
 // (a macro, not a lambda: loaders captured by reference end up in scratch memory)
 #define MQ_GEMM_FETCH(k0)                                       \
   do {                                                          \
     if (FAST) {                                                 \
       la.load_fast(A, g.sam, g.sak, m0, (k0), tid);             \
       lb.load_fast(B, g.sbn, g.sbk, n0, (k0), tid);             \
+      for (int s_ = 1; s_ < nsum; ++s_) lb.add_fast(B + s_ * g.bsum_stride, g.sbn, g.sbk, n0, (k0), tid); \
     } else {                                                    \
       la.load(A, g.sam, g.sak, m0, g.M, (k0), ke, vecA, tid);   \
       lb.load(B, g.sbn, g.sbk, n0, g.N, (k0), ke, vecB, tid);   \

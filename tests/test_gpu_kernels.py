@@ -139,7 +139,7 @@ def _spd(C, seed, n=None):
     return H
 
 
-@pytest.mark.parametrize("C", [128, 256, 384, 896, 1024])
+@pytest.mark.parametrize("C", [128, 256, 384, 896, 1024, 2432])
 def test_factor_vs_torch_chain(dev, C):
     _say(f"factor C={C}")
     H = _spd(C, C)
