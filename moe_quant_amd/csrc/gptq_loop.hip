@@ -4,18 +4,21 @@
 // memory row), so a wavefront that gives one lane to each output row reads and writes fully coalesced.
 // Rows of W never interact, so there is no grid-wide synchronisation anywhere.
 //
-//   per block of <=128 columns [i1, i2):
-//     gptq_block_kernel : each lane keeps its row's 128 block weights in registers, walks the columns
-//                         in order (quantize -> dequantize -> error -> fused-multiply-add of the error
-//                         into the remaining block columns, multiplier U[j,k] wave-uniform via scalar
-//                         loads), and leaves codes, dequantized weights and the error block in memory.
-//     trailing update   : Wt[i2:, :] += U[i1:i2, i2:]^T * E   as an fp32 MFMA GEMM (gemm_f32.hip).
+//   one launch per block b of <=128 columns [i1, i2), two kinds of workgroups:
+//     column workgroups : 64 rows each.  They first bring their 128 columns up to date with the previous
+//                         block's errors (a 128x64x128 product on the matrix cores), then walk the columns in
+//                         order (quantize -> dequantize -> error -> fused-multiply-add of the error into the
+//                         remaining block columns) and leave codes, dequantized weights and the error block.
+//     trailing tiles    : Wt[i2:, :] += U[prev block, i2:]^T * E_prev, the previous block's lazy-batch update
+//                         of everything beyond block b, as 128x128 fp32 MFMA tiles (gemm_f32_tile.hpp).
+//   The sequential walk of block b thus overlaps the bulk of block b-1's trailing update; the error block is
+//   double-buffered.
 //
 // Arithmetic per column is the reference's: q = clamp(floor(x/s + z + 0.5), 0, maxq) with IEEE division,
 // y = round_to(dtype)((q - z) * s), e = y - x, w_k = fma(U[j,k], e, w_k).
 #include <hip/hip_fp16.h>
 
-#include "common.hpp"
+#include "gemm_f32_tile.hpp"
 
 namespace {
 
@@ -41,12 +44,21 @@ struct LoopArgs {
   float qzero_const, maxq;
   int rd;
   uint8_t* Qt;
-  float* E;
+  float* E;            // errors of this block (out)
+  const float* Eprev;  // errors of the previous block (nullable), nbprev columns of them
+  int nbprev;
 };
 
 constexpr int MB = 16;       // micro-block: columns walked with weights in registers
 constexpr int WSTRIDE = 64;  // weight tile in LDS is [column][lane]
-constexpr int UL = 132;      // pitch of the U block in LDS (16-byte aligned rows)
+
+// The 128x128 block of U in LDS: only the 16x16 micro-blocks on or above the diagonal are kept (36 of 64,
+// 36 KB), row-major inside a micro-block, so that this kernel and a 128x128 GEMM tile need the same LDS.
+__device__ __forceinline__ int ut_off(int j, int k) {
+  const int jb = j >> 4, kb = k >> 4;
+  return ((jb * (17 - jb)) / 2 + (kb - jb)) * 256 + (j & 15) * 16 + (k & 15);
+}
+constexpr int UT_FLOATS = 36 * 256;
 
 typedef const int __attribute__((address_space(4))) * cint_p;  // constant address space: scalar loads
 
@@ -63,11 +75,17 @@ typedef const int __attribute__((address_space(4))) * cint_p;  // constant addre
 // use: the kernel is built from branch-free unrolled blocks for that reason (ROWMAP / QZERO are template
 // flags, the rounding mode is a select).
 template <bool FULL, bool ROWMAP, bool QZERO>
-__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int nb) {
+__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int nb, int col_wgs, GemmF32 g, int tiles_n,
+                                                        int vecA, int vecB) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  if ((int)blockIdx.x >= col_wgs) {  // a tile of the previous block's trailing update
+    const int idx = blockIdx.x - col_wgs;
+    gemmf32::tile_body<false, false>(g, idx / tiles_n, idx % tiles_n, 0, reinterpret_cast<float*>(smem), vecA, vecB);
+    return;
+  }
   float* tile = reinterpret_cast<float*>(smem);  // [B][WSTRIDE]
-  float* ut = tile + B * WSTRIDE;                // [B][UL]
-  float* esh = ut + B * UL;                      // [MB][WSTRIDE] errors of the current micro-block
+  float* ut = tile + B * WSTRIDE;                // packed upper micro-blocks of the U block
+  float* esh = ut + UT_FLOATS;                   // [MB][WSTRIDE] errors of the current micro-block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r0 = blockIdx.x * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
@@ -80,6 +98,56 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
     for (int k = 0; k < 32; ++k) t[k] = (FULL || wave * 32 + k < nb) ? wp[(long)(wave * 32 + k) * a.ldw] : 0.f;
 #pragma unroll
     for (int k = 0; k < 32; ++k) tile[(wave * 32 + k) * WSTRIDE + lane] = t[k];
+  }
+  if (a.Eprev) {
+    // The previous block's errors, folded into this block's columns:
+    //   tile[c][row] += sum_k U[i1-nbprev+k, i1+c] * Eprev[k][row].
+    // Wavefront w takes columns 32w..32w+31 and all 64 rows: two 32x32 accumulators.  The errors (shared by the
+    // four wavefronts) are staged in the LDS area the U block will occupy afterwards; the U operand comes
+    // straight from memory in MFMA layout (lane = column, the two k of an instruction in the two lane halves),
+    // every load issued before the first product.
+    float* es = ut;  // [nbprev][64]
+    for (int idx = tid; idx < a.nbprev * 16; idx += 256) {
+      const int k = idx >> 4, r4 = (idx & 15) << 2;
+      const float* q = a.Eprev + (long)k * a.R;
+      float4 v;
+      if (r0 + r4 + 3 < a.R && ((a.R & 3) == 0)) {
+        v = *reinterpret_cast<const float4*>(q + r0 + r4);
+      } else {
+        v.x = q[min(r0 + r4 + 0, a.R - 1)];
+        v.y = q[min(r0 + r4 + 1, a.R - 1)];
+        v.z = q[min(r0 + r4 + 2, a.R - 1)];
+        v.w = q[min(r0 + r4 + 3, a.R - 1)];
+      }
+      *reinterpret_cast<float4*>(&es[k * 64 + r4]) = v;
+    }
+    const int m = lane & 31, slot = lane >> 5;
+    const int col = FULL ? (i1 + wave * 32 + m) : min(i1 + wave * 32 + m, a.C - 1);
+    const float* __restrict__ Uo = a.U + (long)(i1 - a.nbprev) * a.ldu + col;
+    float av[B / 2];
+#pragma unroll
+    for (int t = 0; t < B / 2; ++t) {
+      const int k = 2 * t + slot;
+      const float v = Uo[(long)min(k, a.nbprev - 1) * a.ldu];
+      av[t] = k < a.nbprev ? v : 0.f;
+    }
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < B / 2; ++t) {
+      const int k = min(2 * t + slot, a.nbprev - 1);  // rows past nbprev meet a zero multiplier
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], es[k * 64 + m], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], es[k * 64 + 32 + m], acc1, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int c = wave * 32 + 8 * (v >> 2) + 4 * slot + (v & 3);
+      tile[c * WSTRIDE + m] += acc0[v];
+      tile[c * WSTRIDE + 32 + m] += acc1[v];
+    }
+    __syncthreads();  // es is about to be overwritten by the U block
   }
   {
     const float* __restrict__ Ub = a.U + (long)i1 * a.ldu + i1;
@@ -96,12 +164,12 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
       for (int u = 0; u < 16; ++u) {
         const int idx = tid + u * 256;
         const int j = idx >> 5, k = (idx & 31) << 2;
-        *reinterpret_cast<float4*>(&ut[j * UL + k]) = v[u];
+        if ((k >> 4) >= (j >> 4)) *reinterpret_cast<float4*>(&ut[ut_off(j, k)]) = v[u];
       }
     } else {
       for (int idx = tid; idx < B * B; idx += 256) {
         const int j = idx >> 7, k = idx & 127;
-        ut[j * UL + k] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
+        if ((k >> 4) >= (j >> 4)) ut[ut_off(j, k)] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
       }
     }
   }
@@ -127,7 +195,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
       for (int J = 0; J < MB; ++J)
 #pragma unroll
         for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
-          um[J][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + J) * UL + c0 + 4 * t4]);
+          um[J][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, c0 + 4 * t4)]);
 #pragma unroll
       for (int J = 0; J < MB; ++J) {
         const float s = sc[J], z = zz[J];
@@ -168,7 +236,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         for (int jj = 0; jj < 4; ++jj)
 #pragma unroll
           for (int t4 = 0; t4 < MB / 4; ++t4)
-            ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[(c0 + jj) * UL + k0 + 4 * t4]);
+            ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + jj, k0 + 4 * t4)]);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           if (g < 3) {
@@ -177,7 +245,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
 #pragma unroll
               for (int t4 = 0; t4 < MB / 4; ++t4)
                 ug[(g + 1) & 1][jj][t4] =
-                    *reinterpret_cast<const float4*>(&ut[(c0 + 4 * (g + 1) + jj) * UL + k0 + 4 * t4]);
+                    *reinterpret_cast<const float4*>(&ut[ut_off(c0 + 4 * (g + 1) + jj, k0 + 4 * t4)]);
           }
 #pragma unroll
           for (int jj = 0; jj < 4; ++jj) {
@@ -200,7 +268,8 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   }
 }
 
-constexpr size_t BLOCK_SMEM = (size_t)(B * WSTRIDE + B * UL + MB * WSTRIDE) * sizeof(float);
+constexpr size_t COL_SMEM = (size_t)(B * WSTRIDE + UT_FLOATS + MB * WSTRIDE) * sizeof(float);
+constexpr size_t BLOCK_SMEM = COL_SMEM > gemmf32::SMEM_BYTES ? COL_SMEM : gemmf32::SMEM_BYTES;
 
 template <bool ROWMAP, bool QZERO>
 int run_loop(const LoopArgs& a, int block, hipStream_t st) {
@@ -213,21 +282,33 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
     attr_done = true;
   }
-  for (int i1 = 0; i1 < a.C; i1 += block) {
+  LoopArgs la = a;
+  int blk = 0, nbprev = 0;
+  for (int i1 = 0; i1 < a.C; i1 += block, ++blk) {
     const int i2 = (i1 + block < a.C) ? i1 + block : a.C;
     const int nb = i2 - i1;
+    la.E = a.E + (long)(blk & 1) * B * a.R;
+    la.Eprev = blk ? a.E + (long)((blk + 1) & 1) * B * a.R : nullptr;
+    la.nbprev = nbprev;
+    // the previous block's update of everything beyond this block: Wt[i2+m, r] += sum_j U[i1-nbprev+j, i2+m] * Eprev[j, r]
+    GemmF32 g{a.U + (long)(i1 - nbprev) * a.ldu + i2, la.Eprev, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw,
+              a.C - i2, a.R, nbprev, 1.f, 1.f, 0, 0, 1, 0, 0, 0};
+    int tiles = 0, tiles_n = 1, vecA = 0, vecB = 0;
+    if (blk && i2 < a.C) {
+      tiles_n = (a.R + gemmf32::BN - 1) / gemmf32::BN;
+      tiles = ((a.C - i2 + gemmf32::BM - 1) / gemmf32::BM) * tiles_n;
+      vecA = mq_gemm_operand_aligned(g.A, g.sak, 0);
+      vecB = mq_gemm_operand_aligned(g.B, g.sbk, 0);
+    }
     if (nb == B)
-      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid), dim3(256), BLOCK_SMEM, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid + tiles), dim3(256), BLOCK_SMEM, st, la, i1,
+                         nb, grid, g, tiles_n, vecA, vecB);
     else
-      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid), dim3(256), BLOCK_SMEM, st, a, i1, nb);
+      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid + tiles), dim3(256), BLOCK_SMEM, st, la, i1,
+                         nb, grid, g, tiles_n, vecA, vecB);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
-    if (i2 < a.C) {
-      // Wt[i2+m, r] += sum_j U[i1+j, i2+m] * E[j, r]
-      GemmF32 g{a.U + (long)i1 * a.ldu + i2, a.E, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw,
-                a.C - i2, a.R, nb, 1.f, 1.f, 0, 0, 1, 0, 0, 0};
-      if ((rc = mq_launch_gemm_f32(g, st)) != MQ_OK) return rc;
-    }
+    nbprev = nb;
   }
   return MQ_OK;
 }
@@ -241,7 +322,7 @@ extern "C" int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, l
   if (ldw < R || ldu < C || ld_scale < R) return MQ_ERR_ARG;
   if (round_dtype < 0 || round_dtype > 2) return MQ_ERR_ARG;
   if (block <= 0 || block > B) block = B;  // wider blocks only reassociate the trailing sums
-  LoopArgs a{Wt, ldw, C, R, U, ldu, scale, ld_scale, scale_row, qzero, qzero_const, maxq, round_dtype, Qt, E};
+  LoopArgs a{Wt, ldw, C, R, U, ldu, scale, ld_scale, scale_row, qzero, qzero_const, maxq, round_dtype, Qt, E, nullptr, 0};
   hipStream_t st = (hipStream_t)stream;
   if (scale_row) return qzero ? run_loop<true, true>(a, block, st) : run_loop<true, false>(a, block, st);
   return qzero ? run_loop<false, true>(a, block, st) : run_loop<false, false>(a, block, st);
