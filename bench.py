@@ -216,6 +216,10 @@ def main():
     codes = ops.untranspose_codes(Qt)
     t_pack_rc = timed(lambda: ops.pack_int4(codes), reps=10)
 
+    pts = torch.linspace(1, 0.2, 100, dtype=torch.float32, device=dev)
+    s_try = s_rg.clone()
+    t_mse = timed(lambda: ops.mse_scale_sym_(Wd, 128, pts, s_try, None, 8.0, 15.0, 2.4, torch.bfloat16))
+
     flop_syrk = n * C * (C + 1)
     flop_factor = (2.0 / 3.0) * C**3
     flop_loop = R * C * (C - 1)
@@ -226,6 +230,7 @@ def main():
         "gptq_loop_ms": round(t_loop, 4),
         "pack_from_loop_codes_ms": round(t_pack, 4),
         "pack_int4_ms": round(t_pack_rc, 4),
+        "mse_scale_search_ms_not_in_step": round(t_mse, 4),
         "hessian_syrk_tflops": round(flop_syrk / t_syrk / 1e9, 2),
         "hessian_syrk_frac_bf16_peak": round(flop_syrk / t_syrk / 1e9 / PEAK_BF16_MFMA, 4),
         "factor_tflops": round(flop_factor / t_factor / 1e9, 2),

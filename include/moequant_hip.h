@@ -109,6 +109,19 @@ int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, 
 int mq_quant_grid_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size, int bits,
                       const uint8_t* dead_cols, int round_dtype, float* scale_rg, float* scale_gr, void* stream);
 
+/* Scale search on top of the scales above.  Replaces mse_scale / mse_scale_triton_kernel, src/quant_utils.py:104-192,
+ * as called from get_quantization_grid, :221-232 (QuantizationScale.MSE):
+ *   for every (row, group): candidates s_i = round_to(round_dtype)(scale * p[i]), i < P <= 256;
+ *   loss_i = sum over the group of |dq_i(q_i(w)) - w|^norm with q = clamp(floor(w/s_i + qzero + 0.5), 0, maxq),
+ *   dq = round_to(round_dtype)((q - qzero) * s_i);  scale <- s_best, best = the LAST index of minimal loss
+ *   (tl.argmin(..., tie_break_left=False)).
+ *   p : P fp32 shrink factors on the device (the reference builds them with torch.linspace(1, 0.2, 100)).
+ *   scale_rg : R x G fp32, in (from mq_quant_grid_sym) and out;  scale_gr (nullable): transposed copy, G x R.
+ */
+int mq_mse_scale_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size, const uint8_t* dead_cols,
+                     const float* p, int P, float qzero, float maxq, float norm, int round_dtype, float* scale_rg,
+                     float* scale_gr, void* stream);
+
 /* Wt[j, r] = fp32(W[r, perm[j]]), 0 for dead columns.  Replaces `self.W.clone().float()`,
  * `self.W[:, pruned_ids] = 0` (src/gptq.py:149-152) and `self.W.transpose(-2, -1)[perm]` (src/gptq.py:192).
  * perm nullable = identity. */

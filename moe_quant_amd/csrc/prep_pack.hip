@@ -53,6 +53,88 @@ __global__ __launch_bounds__(256) void grid_sym_kernel(const void* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Scale search: for every (row, group) try the shrunken scales round(s0 * p_i) and keep the one whose
+// quantize-dequantize error sum |dq - x|^norm is smallest, the last one among equals.
+// One wavefront per group, one LANE PER CANDIDATE (up to 4 per lane): the group's weights are handed round as
+// wave-uniform values (v_readlane), every lane runs the quantizer of the column loop on them for its own
+// candidate scales and keeps its own running sums, so no reduction is needed until the final arg-min.
+// |d|^norm = exp2(norm * log2|d|), which is 0 for d = 0 like the reference's exp(log|d| * norm).
+// ---------------------------------------------------------------------------------------------
+constexpr int MSE_NC = 4;  // candidates per lane: P <= 256
+
+__device__ __forceinline__ float round_sel(float x, int rd) {
+  const float b = round_to_bf16(x);
+  const float h = __half2float(__float2half_rn(x));
+  return rd == DT_BF16 ? b : (rd == DT_F16 ? h : x);
+}
+
+__global__ __launch_bounds__(256) void mse_scale_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C, int g,
+                                                        int G, const uint8_t* __restrict__ dead, const float* __restrict__ p,
+                                                        int P, float qzero, float maxq, float norm, int rd,
+                                                        float* __restrict__ scale_rg, float* __restrict__ scale_gr) {
+  const int lane = threadIdx.x & 63;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)R * G) return;
+  const int row = (int)(item / G), grp = (int)(item - (long)row * G);
+  const float s0 = scale_rg[(long)row * G + grp];
+  float sp[MSE_NC], loss[MSE_NC];
+#pragma unroll
+  for (int c = 0; c < MSE_NC; ++c) {
+    const int idx = lane + 64 * c;
+    sp[c] = round_sel(s0 * p[min(idx, P - 1)], rd);
+    loss[c] = 0.f;
+  }
+  const int c0 = grp * g;
+  for (int e0 = 0; e0 < g; e0 += 64) {
+    const int col = c0 + e0 + lane;
+    float xv = 0.f;
+    if (e0 + lane < g) {
+      xv = load_as_f32(W, (long)row * ldw + col, wdt);
+      if (dead && dead[col]) xv = 0.f;
+    }
+    const int cnt = min(64, g - e0);
+#pragma unroll 4
+    for (int j = 0; j < cnt; ++j) {
+      const float x = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xv), j));
+#pragma unroll
+      for (int c = 0; c < MSE_NC; ++c) {
+        if (64 * c < P) {  // wave-uniform
+          float q = floorf(x / sp[c] + qzero + 0.5f);
+          q = fminf(fmaxf(q, 0.f), maxq);
+          const float d = fabsf(round_sel((q - qzero) * sp[c], rd) - x);
+          loss[c] += __builtin_amdgcn_exp2f(norm * __builtin_amdgcn_logf(d));
+        }
+      }
+    }
+  }
+  // arg-min with the larger index winning ties: inside the lane, then across the wavefront
+  float bl = __builtin_inff();
+  int bi = -1;
+#pragma unroll
+  for (int c = 0; c < MSE_NC; ++c) {
+    const int idx = lane + 64 * c;
+    if (idx < P && (loss[c] < bl || (loss[c] == bl && idx > bi))) {
+      bl = loss[c];
+      bi = idx;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ol = __shfl_xor(bl, off, 64);
+    const int oi = __shfl_xor(bi, off, 64);
+    if (oi >= 0 && (bi < 0 || ol < bl || (ol == bl && oi > bi))) {
+      bl = ol;
+      bi = oi;
+    }
+  }
+  if (lane == 0) {
+    const float s = round_sel(s0 * p[max(bi, 0)], rd);
+    scale_rg[(long)row * G + grp] = s;
+    if (scale_gr) scale_gr[(long)grp * R + row] = s;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Wt[j, r] = W[r, perm[j]] as fp32 (0 for dead columns).  64x64 tiles through LDS.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void prepare_wt_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C,
@@ -199,6 +281,19 @@ extern "C" int mq_quant_grid_sym(const void* W, int w_dtype, long ldw, int R, in
   const long items = (long)R * G;
   hipLaunchKernelGGL(grid_sym_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, W, w_dtype,
                      ldw, R, C, group_size, G, dead_cols, two_over_maxq, round_dtype, scale_rg, scale_gr);
+  return mq_check_launch();
+}
+
+extern "C" int mq_mse_scale_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size,
+                                const uint8_t* dead_cols, const float* p, int P, float qzero, float maxq, float norm,
+                                int round_dtype, float* scale_rg, float* scale_gr, void* stream) {
+  if (!W || !p || !scale_rg || R <= 0 || C <= 0 || group_size <= 0 || C % group_size != 0) return MQ_ERR_ARG;
+  if (w_dtype < 0 || w_dtype > 2 || round_dtype < 0 || round_dtype > 2 || ldw < C) return MQ_ERR_ARG;
+  if (P <= 0 || P > 64 * MSE_NC) return MQ_ERR_ARG;
+  const int G = C / group_size;
+  const long items = (long)R * G;
+  hipLaunchKernelGGL(mse_scale_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, W, w_dtype, ldw,
+                     R, C, group_size, G, dead_cols, p, P, qzero, maxq, norm, round_dtype, scale_rg, scale_gr);
   return mq_check_launch();
 }
 

@@ -48,10 +48,11 @@ class GPTQ:
         self.rel_damp = rel_damp
         self.block_size = block_size or self.d_col
         self.quantization_order = QuantizationOrder(quantization_order)
+        # "absmax" or "mse".  The reference compares this string with an Enum member (src/quant_utils.py:221),
+        # which never matches, so its scale search is dead code; here "mse" runs the search.
+        if quantization_scale not in ("absmax", "mse"):
+            raise ValueError(f"quantization_scale must be 'absmax' or 'mse', got {quantization_scale!r}")
         self.quantization_scale = quantization_scale
-        if quantization_scale != "absmax":
-            # the reference compares this string with an Enum member, which never matches: absmax runs
-            warnings.warn(f"quantization_scale={quantization_scale!r} behaves as 'absmax', as in MoE-Quant")
         self.W_device = self.W.device
         self.W_dtype = self.W.dtype
         self.W_shape = self.W.shape
@@ -242,6 +243,10 @@ class GPTQ:
         W, dead = self._kernel_weights()
         # per-group scales from the un-updated weights (src/gptq.py:171-178): compact (R,G) and (G,R)
         scale_rg, scale_gr = ops.quant_grid_sym(W, group_size, bits, dtype, dead_cols=dead)
+        if self.quantization_scale == "mse":  # src/quant_utils.py:221-232 with its default search grid
+            points = torch.linspace(1, 0.2, 100, dtype=torch.float32, device=device)
+            ops.mse_scale_sym_(W, group_size, points, scale_rg, scale_gr, float(2 ** (bits - 1)), float(2**bits - 1), 2.4,
+                               dtype, dead_cols=dead)
         tied = self.tied_gptq_handle
         perm = perm_inv = perm_i32 = perm_inv_i32 = None
         if self.quantization_order == QuantizationOrder.ACTIVATION:

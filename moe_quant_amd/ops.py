@@ -189,6 +189,28 @@ def quant_grid_sym(W: Tensor, group_size: int, bits: int, round_dtype, dead_cols
     return s_rg, s_gr
 
 
+def mse_scale_sym_(W: Tensor, group_size: int, p: Tensor, scale_rg: Tensor, scale_gr: Optional[Tensor], qzero: float,
+                   maxq: float, norm: float, round_dtype, dead_cols: Optional[Tensor] = None) -> Tensor:
+    """In place on scale_rg (R,G) fp32 (and its transposed copy scale_gr): the scale search over shrink factors p."""
+    _dev(W, p, scale_rg, scale_gr, dead_cols)
+    lib = _lib.load()
+    R, C = W.shape
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    G = C // group_size
+    if scale_rg.dtype != torch.float32 or scale_rg.shape != (R, G) or not scale_rg.is_contiguous():
+        raise ValueError("scale_rg must be a contiguous (R,G) fp32 tensor")
+    if scale_gr is not None and (scale_gr.dtype != torch.float32 or scale_gr.shape != (G, R) or not scale_gr.is_contiguous()):
+        raise ValueError("scale_gr must be a contiguous (G,R) fp32 tensor")
+    if p.dtype != torch.float32 or p.dim() != 1 or not p.is_contiguous():
+        raise ValueError("p must be a contiguous fp32 vector")
+    rc = lib.mq_mse_scale_sym(W.data_ptr(), _dt(W.dtype), W.stride(0), R, C, group_size, _p(dead_cols), p.data_ptr(),
+                              p.numel(), float(qzero), float(maxq), float(norm), _dt(round_dtype), scale_rg.data_ptr(),
+                              _p(scale_gr), _stream(W))
+    check(rc, "mq_mse_scale_sym")
+    return scale_rg
+
+
 def prepare_wt(W: Tensor, perm: Optional[Tensor] = None, dead_cols: Optional[Tensor] = None) -> Tensor:
     _dev(W, perm, dead_cols)
     lib = _lib.load()

@@ -54,6 +54,21 @@ def find_quantization_meta(x: Tensor, bit_width: int, symmetric: bool = False, d
 
 
 @torch.no_grad()
+def mse_scale(x: Tensor, p: Tensor, scale: Tensor, qzero: Tensor, maxq: Tensor, dtype: torch.dtype = None,
+              norm: float = 2.4) -> Tensor:
+    """src/quant_utils.py:143-192: x (..., g) weights of each group, p (P,) shrink factors, scale/qzero (...);
+    `scale` is modified in place and returned.  Symmetric grids only: one zero point for all groups."""
+    assert x.is_contiguous() and p.is_contiguous() and scale.is_contiguous() and qzero.is_contiguous()
+    g = x.shape[-1]
+    x2 = x.reshape(-1, g)
+    z = float(qzero.reshape(-1)[0].item()) if qzero.numel() else 0.0
+    sc = scale.reshape(-1, 1).float().contiguous()
+    ops.mse_scale_sym_(x2, g, p.float().contiguous(), sc, None, z, float(maxq.item()), norm, dtype)
+    scale.copy_(sc.reshape(scale.shape).to(scale.dtype))
+    return scale
+
+
+@torch.no_grad()
 def get_quantization_grid(
     weight: Tensor,
     group_size: int,
@@ -66,14 +81,16 @@ def get_quantization_grid(
     quant_norm: float = 2.4,
 ):
     """src/quant_utils.py:195-240: returns (scale (...,C), qzero (...,C), maxq ()) replicated per column."""
-    if quantization_scale == QuantizationScale.MSE:
-        raise NotImplementedError("MSE scale search is outside this engine's scope")
-    if isinstance(quantization_scale, str) and quantization_scale != "absmax":
-        # the reference compares this string to an Enum, which is never equal: absmax is what it runs
-        warnings.warn(f"quantization_scale={quantization_scale!r} behaves as 'absmax', as in MoE-Quant")
+    # The reference tests `quantization_scale == QuantizationScale.MSE`, which a plain string never satisfies
+    # (src/gptq.py:47 stores the string): its search is unreachable from the GPTQ class.  Here both the enum
+    # member and the string "mse" select it.
+    mse = quantization_scale == QuantizationScale.MSE or quantization_scale == "mse"
     group_size = group_size or weight.shape[-1]
     w = weight.unflatten(dim=-1, sizes=(-1, group_size))
     scale, qzero, maxq = find_quantization_meta(w, bits, symmetric, dtype)
+    if mse:
+        search_points = torch.linspace(1, quant_max_shrink, quant_n_grid, dtype=torch.float32, device=weight.device)
+        scale = mse_scale(w.contiguous(), search_points, scale.contiguous(), qzero, maxq, dtype, quant_norm)
     scale = scale.repeat_interleave(group_size, dim=-1)
     qzero = qzero.repeat_interleave(group_size, dim=-1)
     assert weight.shape == scale.shape == qzero.shape and maxq.shape == ()

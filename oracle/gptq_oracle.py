@@ -21,6 +21,11 @@ pinned by closed forms / invariants / brute force in tests/test_oracle_*.py:
                               round trip.  compressed_tensors is absent from this image and un-pinned
                               by the reference (no version, no tests) -> "parity unpinned" beyond that.
   dequantize / relative_mse . closed form; tr(dH d^T) = (2/n)||X d^T||_F^2 against fp64 matmul
+  mse_scale ................. brute force over the candidates in fp64 on tiny groups with well-separated
+                              losses; the chosen candidate never loses to p = 1; all-zero group -> every loss
+                              0 -> the LAST candidate wins (tie_break_left=False); a group that sits exactly
+                              on the 4-bit grid keeps p = 1.  The bits of Triton's log/exp and the order of
+                              its group sum decide near-ties between candidates: "parity unpinned" there.
 
 Unpinnable by any means: torch.argsort tie order (unstable sort) and the exact
 bits of Triton's fma / division on a GPU.
@@ -103,15 +108,51 @@ def find_quantization_meta(x: Tensor, bit_width: int, dtype: Optional[torch.dtyp
     return scale, qzero, maxq
 
 
-def quantization_grid(W: Tensor, group_size: Optional[int], bits: int, dtype: Optional[torch.dtype]):
-    """Compact grid: scale (R,G) fp32 (bf16-exact), qzero (R,G), maxq () -- src/quant_utils.py:213-220."""
+def quantization_grid(W: Tensor, group_size: Optional[int], bits: int, dtype: Optional[torch.dtype],
+                      mse: bool = False, max_shrink: float = 0.2, n_grid: int = 100, norm: float = 2.4):
+    """Compact grid: scale (R,G) fp32 (bf16-exact), qzero (R,G), maxq () -- src/quant_utils.py:213-232.
+    mse=True adds the scale search of :221-232 (what QuantizationScale.MSE selects)."""
     g = group_size or W.shape[-1]
-    return find_quantization_meta(W.unflatten(-1, (-1, g)), bits, dtype)
+    x = W.unflatten(-1, (-1, g))
+    scale, qzero, maxq = find_quantization_meta(x, bits, dtype)
+    if mse:
+        scale = mse_scale(x.contiguous(), search_points(max_shrink, n_grid), scale, qzero, maxq, dtype, norm)
+    return scale, qzero, maxq
 
 
 def replicate_grid(scale: Tensor, qzero: Tensor, group_size: int):
     """(R,G) -> (R,C) as src/quant_utils.py:234-235."""
     return scale.repeat_interleave(group_size, dim=-1), qzero.repeat_interleave(group_size, dim=-1)
+
+
+def mse_scale(x: Tensor, p: Tensor, scale: Tensor, qzero: Tensor, maxq: Tensor, dtype: Optional[torch.dtype] = None,
+              norm: float = 2.4, chunk: int = 4096) -> Tensor:
+    """Scale search of src/quant_utils.py:104-192: x (..., g) fp32, p (P,) shrink factors, scale/qzero (...).
+    For every group the candidate scale round_fp(scale*p_i) minimising sum |dq(q(x)) - x|^norm wins, the last one
+    among equals (tl.argmin(..., tie_break_left=False), :138); returns round_fp(scale * p[best]) (:140).
+    |d|^norm is evaluated as exp(log|d| * norm) like tl_pow (:26-27); the quantizer is the Triton one
+    (floor(v + 0.5), :30-49).  `scale` is not modified (the reference overwrites it in place)."""
+    g = x.shape[-1]
+    xs = x.reshape(-1, g)
+    sc = scale.reshape(-1)
+    qz = qzero.reshape(-1)
+    out = torch.empty_like(sc)
+    P = p.numel()
+    for s0 in range(0, xs.shape[0], chunk):
+        xb = xs[s0 : s0 + chunk][:, None, :]  # (B, 1, g)
+        sp = round_fp(sc[s0 : s0 + chunk, None] * p[None, :], dtype)[:, :, None]  # (B, P, 1)  :135
+        zb = qz[s0 : s0 + chunk, None, None]
+        q = torch.floor(xb / sp + zb + 0.5).clamp(torch.zeros_like(maxq), maxq)  # tl_quantize
+        dq = round_fp((q - zb) * sp, dtype)  # tl_dequantize
+        loss = ((dq - xb).abs().log() * norm).exp().sum(dim=-1)  # (B, P)  :137
+        best = (P - 1) - torch.argmin(loss.flip(-1), dim=-1)  # last index among equal minima
+        out[s0 : s0 + chunk] = round_fp(sc[s0 : s0 + chunk] * p[best], dtype)  # :140
+    return out.reshape(scale.shape)
+
+
+def search_points(max_shrink: float = 0.2, n_grid: int = 100) -> Tensor:
+    """src/quant_utils.py:222."""
+    return torch.linspace(1, max_shrink, n_grid, dtype=torch.float32)
 
 
 def quantize(x: Tensor, scale: Tensor, qzero: Tensor, maxq: Tensor, half_up: bool = True) -> Tensor:
@@ -234,13 +275,14 @@ def quantize_linear(
     dtype: Optional[torch.dtype] = None,
     half_up: bool = True,
     inverse_dtype=torch.float32,
+    mse: bool = False,
 ):
     """Returns dict(qweight u8 (R,C), scale (R,G), zero (R,G), U, perm, H (damped, permuted), ok)."""
     dtype = dtype or W.dtype
     R, C = W.shape
     H, W32, zero_samples, nan_h = quantization_pre_step(H, W)
     g = group_size or C
-    scale_g, zero_g, maxq = quantization_grid(W32, g, bits, dtype)  # src/gptq.py:171-178
+    scale_g, zero_g, maxq = quantization_grid(W32, g, bits, dtype, mse=mse)  # src/gptq.py:171-178
     scale, zero = replicate_grid(scale_g, zero_g, g)
     perm, perm_inv = act_order_perm(H, act_order)
     H = H[perm][:, perm]  # src/gptq.py:187

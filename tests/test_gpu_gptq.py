@@ -225,6 +225,28 @@ def test_tied_handles_share_hessian_and_factor(dev):
     up.reset()
 
 
+def test_mse_scale_option_end_to_end(dev):
+    """quantization_scale="mse": scales from the search, then the same loop.  Where a scale differs from the oracle's
+    (near-ties of the search) that group's codes differ too, so the gate is on the layer-output error."""
+    case = synth.config1(0.125)
+    h = GPTQ(_layer(case.W, dev), 128, True, 0.01, 128, quantization_scale="mse")
+    h.update(case.X.to(dev))
+    q, s, z = h.quantize(4)
+    Href, _ = O.hessian_update(None, 0, case.X)
+    ref = O.quantize_linear(case.W, Href.clone(), mse=True)
+    same = (s.cpu() == ref["scale"]).float().mean().item()
+    H64 = O.hessian_fp64([case.X])
+    Wd = case.W.double()
+    e_hip = O.relative_mse(O.dequantize_linear_weight(q.cpu(), s.cpu(), z.cpu()).double(), Wd, H64).item()
+    e_ref = O.relative_mse(O.dequantize_linear_weight(ref["qweight"], ref["scale"], ref["zero"]).double(), Wd, H64).item()
+    plain = O.quantize_linear(case.W, Href.clone())
+    _say(f"  mse option: scales equal {same:.4f}, rel-mse hip {e_hip:.5e} oracle {e_ref:.5e}")
+    assert same >= 0.97 and abs(e_hip - e_ref) <= 0.01 * e_ref
+    assert (ref["scale"] != plain["scale"]).float().mean().item() > 0.1  # the search is not a no-op here
+    rows = (s.cpu() == ref["scale"]).all(dim=1)  # rows whose scales all agree must agree on (nearly) all codes
+    assert (q.cpu()[rows] == ref["qweight"][rows]).float().mean().item() >= 0.999
+
+
 def test_update_many_equals_update(dev):
     Ws = [synth.weight(64, 512, 60 + i) for i in range(3)]
     Xa = [synth.activations_outlier(400 + 100 * i, 512, 70 + i).to(dev) for i in range(3)]

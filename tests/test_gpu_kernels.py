@@ -393,3 +393,39 @@ def test_pack_bit_exact(dev, R, C):
     assert torch.equal(got, want)
     # round trip
     assert torch.equal(O.unpack_from_int32(got, 4, (R, C)) + 8, q.to(torch.int8))
+
+
+# ---------------------------------------------------------------- scale search (src/quant_utils.py:104-192)
+@pytest.mark.parametrize("R,C,g,dtype", [(256, 512, 128, torch.bfloat16), (64, 384, 64, torch.bfloat16),
+                                         (40, 200, 100, torch.float32), (32, 256, 32, torch.float16)])
+def test_mse_scale_search(dev, R, C, g, dtype):
+    """Scales after the search equal the oracle's except where two candidates' losses tie to within the rounding of
+    log/exp (the kernel uses the hardware's base-2 pair, the oracle torch's natural ones): there the chosen
+    candidate must still be as good as the oracle's."""
+    _say(f"mse scale R={R} C={C} g={g} {dtype}")
+    W = synth.weight(R, C, 11 + R, dtype=dtype)
+    W[:, ::37] *= 3.0  # outliers, so that shrinking pays off in many groups
+    W[3, g : 2 * g] = 0  # an all-zero group: every loss is 0, the last candidate wins
+    p = O.search_points()
+    x = W.float().reshape(R, C // g, g)
+    rd = dtype if dtype != torch.float32 else torch.bfloat16
+    s0, z0, maxq = O.find_quantization_meta(x, 4, rd)
+    want = O.mse_scale(x.contiguous(), p, s0, z0, maxq, rd, 2.4)
+    s_rg, s_gr = ops.quant_grid_sym(W.to(dev), g, 4, rd)
+    assert torch.equal(s_rg.cpu(), s0)
+    ops.mse_scale_sym_(W.to(dev), g, p.to(dev), s_rg, s_gr, 8.0, 15.0, 2.4, rd)
+    got = s_rg.cpu()
+    assert torch.equal(s_gr.cpu(), got.t())
+    same = (got == want).float().mean().item()
+    _say(f"  scales equal to the oracle's: {same:.4f}; moved by the search: {(want != s0).float().mean().item():.3f}")
+    assert same >= 0.97
+    assert torch.equal(got[3, 1], (s0[3, 1] * p[-1]).to(rd).float())
+
+    def loss(sc):
+        q = torch.floor(x / sc[..., None] + 8.5).clamp(0, 15)
+        dq = ((q - 8.0) * sc[..., None]).to(rd).float()
+        return (dq - x).abs().double().pow(2.4).sum(-1)
+
+    lg, lw = loss(got), loss(want)
+    ok = ~torch.isnan(lw)  # fp16 rounds the 1e-12 scale of the all-zero group to 0: 0/0 there
+    assert torch.all(lg[ok] <= lw[ok] * (1 + 1e-4) + 1e-30)

@@ -302,3 +302,69 @@ def test_quantize_linear_end_to_end_properties():
     dq2 = O.dequantize_linear_weight(out2["qweight"], out2["scale"], out2["zero"]).double()
     assert O.relative_mse(dq2, case.W.double(), H64).item() < e_rtn
     assert torch.equal(out2["scale"], s)  # static scales do not depend on the order
+
+
+# ---------------------------------------------------------------- MSE scale search (src/quant_utils.py:104-192)
+def _brute_mse_scale(x, p, scale, qzero, maxq, norm):
+    """Independent restatement in Python floats (fp64) with an explicit loop and an explicit last-minimum rule."""
+    import math
+
+    def bf16(v):
+        return torch.tensor(v, dtype=torch.float32).to(torch.bfloat16).float().item()
+
+    out = []
+    for xi, s0, z in zip(x.tolist(), scale.tolist(), qzero.tolist()):
+        best, best_loss = None, None
+        for pi in p.tolist():
+            sp = bf16(torch.tensor(s0, dtype=torch.float32).mul(torch.tensor(pi, dtype=torch.float32)).item())
+            loss = 0.0
+            for v in xi:
+                q = min(max(math.floor(v / sp + z + 0.5), 0.0), maxq)
+                d = abs(bf16((q - z) * sp) - v)
+                loss += d**norm if d > 0 else 0.0
+            if best_loss is None or loss <= best_loss:
+                best, best_loss = sp, loss
+        out.append(best)
+    return torch.tensor(out)
+
+
+def test_mse_scale_matches_brute_force_on_tiny_groups():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(12, 16, generator=g) * 0.03
+    x[:, 0] *= 4.0  # an outlier per group: shrinking the scale pays off
+    p = O.search_points(0.2, 25)
+    scale, qzero, maxq = O.find_quantization_meta(x, 4, torch.bfloat16)
+    got = O.mse_scale(x, p, scale, qzero, maxq, torch.bfloat16, 2.4)
+    want = _brute_mse_scale(x, p, scale, qzero, maxq.item(), 2.4)
+    assert torch.equal(got, want)
+    assert (got < scale).any()  # the search did move some scales
+
+
+def test_mse_scale_special_cases():
+    p = O.search_points()
+    maxq = torch.tensor(15.0)
+    # all-zero group: every candidate has loss 0, the last one wins (tie_break_left=False)
+    x = torch.zeros(1, 128)
+    scale, qzero, _ = O.find_quantization_meta(x, 4, torch.bfloat16)
+    got = O.mse_scale(x, p, scale, qzero, maxq, torch.bfloat16)
+    assert torch.equal(got, (scale * p[-1]).to(torch.bfloat16).float())
+    # a group that already sits on the grid of its absmax scale: p = 1 has loss 0 and is the only such candidate
+    s0 = torch.tensor([0.015625])
+    x = ((torch.arange(128) % 16).float() - 8.0) * s0
+    x = x[None]  # values (k - 8) * s0, k = 0..15: exactly the 4-bit grid of scale s0
+    x[0, 1] = 7.0 * s0
+    scale = torch.tensor([0.015625])
+    got = O.mse_scale(x, p, scale, torch.tensor([8.0]), maxq, torch.bfloat16)
+    assert torch.equal(got, scale)
+    # the winner never loses to the absmax scale itself
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 128, generator=g) * 0.02
+    scale, qzero, _ = O.find_quantization_meta(x, 4, torch.bfloat16)
+    got = O.mse_scale(x, p, scale, qzero, maxq, torch.bfloat16)
+
+    def loss(sc):
+        q = torch.floor(x / sc[:, None] + 8.5).clamp(0, 15)
+        dq = ((q - 8.0) * sc[:, None]).to(torch.bfloat16).float()
+        return (dq - x).abs().double().pow(2.4).sum(-1)
+
+    assert torch.all(loss(got) <= loss(scale) * (1 + 1e-6))
