@@ -1,8 +1,14 @@
-"""Drop-in for pack_weight of MoE-Quant's pack_quantized_model.py (the compressed_tensors
-"pack-quantized" int32 layout), packed by the HIP kernel."""
+"""Drop-in for the model-independent parts of MoE-Quant's pack_quantized_model.py: pack_weight (the
+compressed_tensors "pack-quantized" int32 layout, packed by the HIP kernel), the quantization_config it writes,
+and the per-block step that swaps quantized linears into a block's state dict and saves one safetensors shard.
+Loading the 163-shard DeepSeek checkpoint, the HF config/tokenizer copies and the FP8 dequantization of the
+untouched tensors stay with the caller."""
 from __future__ import annotations
 
-from typing import Optional
+import json
+import os
+from collections import defaultdict
+from typing import Any, Dict, Iterable, Optional
 
 import torch
 
@@ -43,3 +49,78 @@ def pack_weight(weight: dict, bits: int, sym: bool, group_size: Optional[int] = 
     if not sym:
         out["weight_zero_point"] = weight["zero"]
     return out
+
+
+def prepare_quantization_config(bits: int, group_size: int, quantize_only_experts: bool) -> Dict[str, Any]:
+    """pack_quantized_model.py:78-109 (takes the three values instead of the argparse namespace)."""
+    ignored_modules = ["lm_head"]
+    if quantize_only_experts:
+        ignored_modules += ["re:.*self_attn.*", "re:.*shared_experts.*", r"re:.*mlp\.(gate|up|gate_up|down)_proj.*"]
+    return {
+        "config_groups": {
+            "group_0": {
+                "input_activations": None,
+                "output_activations": None,
+                "targets": ["Linear"],
+                "weights": {
+                    "actorder": None,
+                    "block_structure": None,
+                    "dynamic": False,
+                    "group_size": group_size,
+                    "num_bits": bits,
+                    "observer": "minmax",
+                    "observer_kwargs": {},
+                    "strategy": "group",
+                    "symmetric": True,
+                    "type": "int",
+                },
+            }
+        },
+        "format": "pack-quantized",
+        "ignore": ignored_modules,
+        "kv_cache_scheme": None,
+        "quant_method": "compressed-tensors",
+        "quantization_status": "compressed",
+    }
+
+
+def quantized_layers_by_block(quantized_model_path: str) -> Dict[int, list]:
+    """pack_quantized_model.py:143-147: directory names `model.layers.<idx>.<...>` grouped by block index."""
+    names = defaultdict(list)
+    for layer_name in sorted(os.listdir(quantized_model_path)):
+        if os.path.isdir(os.path.join(quantized_model_path, layer_name)):
+            names[int(layer_name.split(".")[2])].append(layer_name)
+    return names
+
+
+def pack_block_state_dict(block_state_dict: Dict[str, torch.Tensor], quantized_model_path: str, layer_names: Iterable[str],
+                          bits: int, sym: bool, group_size: int) -> Dict[str, torch.Tensor]:
+    """pack_quantized_model.py:186-197: for every quantized linear of the block, `<name>.weight` (and the FP8
+    `<name>.weight_scale_inv`) leave the state dict and weight_packed / weight_shape / weight_scale enter it."""
+    for layer_name in layer_names:
+        weight_state_dict = torch.load(os.path.join(quantized_model_path, layer_name, "quantized_weight.pt"),
+                                       weights_only=True, map_location="cpu")
+        packed = pack_weight(weight_state_dict, bits, sym, group_size)
+        block_state_dict.pop(f"{layer_name}.weight")
+        block_state_dict.pop(f"{layer_name}.weight_scale_inv", None)
+        block_state_dict.update({f"{layer_name}.{k}": v for k, v in packed.items()})
+    return block_state_dict
+
+
+def save_packed_shard(block_state_dict: Dict[str, torch.Tensor], packed_model_path: str, shard_id: int, num_shards: int,
+                      safetensors_index: Dict[str, str]) -> str:
+    """pack_quantized_model.py:199-206: one safetensors file per block, recorded in the weight map."""
+    from safetensors.torch import save_file
+
+    os.makedirs(packed_model_path, exist_ok=True)
+    shard = f"model-{shard_id:05}-of-{num_shards:05}.safetensors"
+    save_file({k: v.contiguous() for k, v in block_state_dict.items()}, os.path.join(packed_model_path, shard))
+    for k in block_state_dict:
+        safetensors_index[k] = shard
+    return shard
+
+
+def save_safetensors_index(packed_model_path: str, safetensors_index: Dict[str, str]) -> None:
+    """pack_quantized_model.py:232-233."""
+    with open(os.path.join(packed_model_path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": safetensors_index}, f)

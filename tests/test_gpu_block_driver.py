@@ -117,3 +117,45 @@ def test_block_driver_against_oracle(dev, tmp_path, tie, only_experts):
     meta = torch.load(os.path.join(save_dir, "metadata.pt"), weights_only=True)
     assert meta == {"bits": 4, "group_size": 128, "quantize_only_experts": only_experts}
     assert block_driver.get_resume_block_idx(save_dir) == block_idx
+
+
+def test_pack_block_after_driver(dev, tmp_path):
+    """quantized_weight.pt files -> packed safetensors shard + index + quantization_config, read back and unpacked."""
+    import json
+
+    from safetensors.torch import load_file
+
+    from moe_quant_amd import pack_quantized_model as P
+
+    torch.manual_seed(0)
+    toy = Toy().to(dev).to(torch.bfloat16)
+    block_idx = 2
+    prefix = f"model.layers.{block_idx}."
+    block = toy.model.layers[block_idx]
+    x = torch.randn(500, HID, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(dev)
+    qdir, pdir = str(tmp_path / "q"), str(tmp_path / "p")
+    block_driver.quantize_block(toy, prefix, lambda: block(x), quantize_only_experts=True, save_dir=qdir)
+    block_driver.save_metadata(qdir, 4, 128, True)
+    meta = torch.load(os.path.join(qdir, "metadata.pt"), weights_only=True)
+    names = P.quantized_layers_by_block(qdir)
+    assert list(names) == [block_idx] and len(names[block_idx]) == 3 * NEXP
+    sd = {f"{prefix}{k}": v.detach().cpu() for k, v in block.state_dict().items()}
+    sd = P.pack_block_state_dict(sd, qdir, names[block_idx], meta["bits"], True, meta["group_size"])
+    index = {}
+    shard = P.save_packed_shard(sd, pdir, block_idx + 2, 6, index)
+    P.save_safetensors_index(pdir, index)
+    back = load_file(os.path.join(pdir, shard))
+    wm = json.load(open(os.path.join(pdir, "model.safetensors.index.json")))["weight_map"]
+    assert set(wm) == set(back) == set(sd)
+    for name in names[block_idx]:
+        blob = torch.load(os.path.join(qdir, name, "quantized_weight.pt"), weights_only=True)
+        assert f"{name}.weight" not in back
+        words, shape = back[f"{name}.weight_packed"], back[f"{name}.weight_shape"]
+        assert words.dtype == torch.int32 and shape.tolist() == list(blob["qweight"].shape)
+        assert torch.equal(O.unpack_from_int32(words, 4, shape.tolist()), blob["qweight"].cpu().to(torch.int8) - 8)
+        assert torch.equal(back[f"{name}.weight_scale"], blob["scale"].cpu())
+    assert f"{prefix}self_attn.o_proj.weight" in back  # untouched tensors travel along
+    cfg = P.prepare_quantization_config(meta["bits"], meta["group_size"], meta["quantize_only_experts"])
+    w = cfg["config_groups"]["group_0"]["weights"]
+    assert cfg["format"] == "pack-quantized" and w["num_bits"] == 4 and w["group_size"] == 128 and w["symmetric"]
+    assert "re:.*shared_experts.*" in cfg["ignore"] and cfg["ignore"][0] == "lm_head"
