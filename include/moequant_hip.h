@@ -169,6 +169,15 @@ int mq_pack_from_qt(const uint8_t* Qt, int R, int C, const int* perm_inv, int32_
 int mq_gemm_f32(const float* A, long sam, long sak, const float* B, long sbk, long sbn, float* C, long ldc, int M,
                 int N, int K, float alpha, float beta, int tri, int ktrim, void* stream);
 
+/* ---- checkpoint ingest: FP8 weights with per-128x128-block inverse scales -> bf16 / fp16 -------------------
+ * Replaces `W.to(dtype)`, `s.to(dtype)` and dequantize_weight_from_fp8, src/quant_utils.py:267-296, in one pass:
+ *   out[r, c] = round_to(out_dtype)( e4m3fn(W[r, c]) * round_to(out_dtype)(scale_inv[r/128, c/128]) ).
+ *   W : R x C bytes (ldw), OCP e4m3fn (torch.float8_e4m3fn); scale_inv : ceil(R/128) x ceil(C/128) fp32 (ld_scale);
+ *   out : R x C 16-bit floats (ldo), out_dtype = MQ_DT_BF16 or MQ_DT_F16.  No padding is needed for ragged edges.
+ */
+int mq_dequant_fp8_block(const uint8_t* W, long ldw, int R, int C, const float* scale_inv, long ld_scale, int out_dtype,
+                         void* out, long ldo, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,7 @@ SIGNATURES = {
     "mq_untranspose_codes": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
     "mq_pack_int4": (_i, [_vp, _l, _i, _i, _vp, _i, _vp, _l, _vp]),
     "mq_pack_from_qt": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
+    "mq_dequant_fp8_block": (_i, [_vp, _l, _i, _i, _vp, _l, _i, _vp, _l, _vp]),
     "mq_gemm_f32": (_i, [_vp, _l, _l, _vp, _l, _l, _vp, _l, _i, _i, _i, _f, _f, _i, _i, _vp]),
 }
 

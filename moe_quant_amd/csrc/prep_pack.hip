@@ -267,6 +267,51 @@ __global__ __launch_bounds__(256) void pack_from_qt_kernel(const uint8_t* __rest
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// FP8 (e4m3fn) checkpoint weights with one fp32 inverse scale per 128x128 block -> bf16 / fp16:
+//   out = round_to(dtype)( fp8_value * round_to(dtype)(scale_inv[block]) ),
+// the value of `W.to(dtype) * s.to(dtype)` (fp8 -> 16-bit float is exact).  16 weights per thread:
+// one 16-byte load, two 16-byte stores.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float e4m3fn_to_f32(uint32_t b) {
+  const uint32_t sign = (b & 0x80u) << 24, e = (b >> 3) & 0xFu, m = b & 7u;
+  float v;
+  if (e == 0) v = (float)m * 0.001953125f;  // subnormal: m * 2^-9
+  else if (e == 15 && m == 7) v = __uint_as_float(0x7fc00000u);
+  else v = __uint_as_float(((e + 120u) << 23) | (m << 20));
+  return __uint_as_float(__float_as_uint(v) | sign);
+}
+
+__device__ __forceinline__ uint16_t to_16bit(float x, int dt) {
+  return dt == DT_BF16 ? f32_to_bf16_bits(x) : __half_as_ushort(__float2half_rn(x));
+}
+
+__global__ __launch_bounds__(256) void dequant_fp8_kernel(const uint8_t* __restrict__ W, long ldw, int R, int C,
+                                                          const float* __restrict__ sinv, long lds, int dt,
+                                                          uint16_t* __restrict__ out, long ldo, int vec) {
+  const int chunks = (C + 15) / 16;
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;
+  if (item >= (long)R * chunks) return;
+  const int r = (int)(item / chunks), c0 = (int)(item - (long)r * chunks) * 16;
+  const float s = round_sel(sinv[(long)(r >> 7) * lds + (c0 >> 7)], dt);  // a 16-chunk never straddles a block
+  const uint8_t* src = W + (long)r * ldw + c0;
+  uint16_t* dst = out + (long)r * ldo + c0;
+  if (vec && c0 + 16 <= C) {
+    const uint4 v = *reinterpret_cast<const uint4*>(src);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const uint32_t lo = (w[k >> 1] >> (16 * (k & 1))) & 0xffu, hi = (w[k >> 1] >> (16 * (k & 1) + 8)) & 0xffu;
+      o[k] = (uint32_t)to_16bit(e4m3fn_to_f32(lo) * s, dt) | ((uint32_t)to_16bit(e4m3fn_to_f32(hi) * s, dt) << 16);
+    }
+    *reinterpret_cast<uint4*>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
+    *reinterpret_cast<uint4*>(dst + 8) = make_uint4(o[4], o[5], o[6], o[7]);
+  } else {
+    for (int k = 0; k < 16 && c0 + k < C; ++k) dst[k] = to_16bit(e4m3fn_to_f32(src[k]) * s, dt);
+  }
+}
+
 }  // namespace
 
 extern "C" int mq_quant_grid_sym(const void* W, int w_dtype, long ldw, int R, int C, int group_size, int bits,
@@ -337,5 +382,17 @@ extern "C" int mq_pack_from_qt(const uint8_t* Qt, int R, int C, const int* perm_
   if (ldo < words) return MQ_ERR_ARG;
   hipLaunchKernelGGL(pack_from_qt_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream, Qt, R,
                      C, perm_inv, out, ldo, words);
+  return mq_check_launch();
+}
+
+extern "C" int mq_dequant_fp8_block(const uint8_t* W, long ldw, int R, int C, const float* scale_inv, long ld_scale,
+                                    int out_dtype, void* out, long ldo, void* stream) {
+  if (!W || !scale_inv || !out || R <= 0 || C <= 0 || ldw < C || ldo < C) return MQ_ERR_ARG;
+  if (out_dtype != DT_BF16 && out_dtype != DT_F16) return MQ_ERR_ARG;
+  if (ld_scale < (C + 127) / 128) return MQ_ERR_ARG;
+  const int vec = ((uintptr_t)W % 16 == 0) && (ldw % 16 == 0) && ((uintptr_t)out % 16 == 0) && (ldo % 8 == 0);
+  const long items = (long)R * ((C + 15) / 16);
+  hipLaunchKernelGGL(dequant_fp8_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, (hipStream_t)stream, W, ldw, R,
+                     C, scale_inv, ld_scale, out_dtype, (uint16_t*)out, ldo, vec);
   return mq_check_launch();
 }

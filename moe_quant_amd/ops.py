@@ -289,6 +289,27 @@ def pack_from_qt(Qt: Tensor, perm_inv: Optional[Tensor] = None) -> Tensor:
     return out
 
 
+def dequant_fp8_block(W: Tensor, scale_inv: Tensor, dtype: torch.dtype) -> Tensor:
+    """W (R,C) torch.float8_e4m3fn, scale_inv (ceil(R/128), ceil(C/128)) any float -> (R,C) bf16/fp16."""
+    _dev(W, scale_inv)
+    lib = _lib.load()
+    if W.dtype != torch.float8_e4m3fn or W.dim() != 2:
+        raise TypeError("W must be a 2-D torch.float8_e4m3fn tensor")
+    if dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("dtype must be bfloat16 or float16")
+    R, C = W.shape
+    if scale_inv.shape != ((R + 127) // 128, (C + 127) // 128):
+        raise ValueError("scale_inv must have one entry per 128x128 block")
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    s = scale_inv.to(torch.float32).contiguous()
+    out = torch.empty(R, C, dtype=dtype, device=W.device)
+    rc = lib.mq_dequant_fp8_block(W.data_ptr(), W.stride(0), R, C, s.data_ptr(), s.stride(0), _dt(dtype), out.data_ptr(),
+                                  out.stride(0), _stream(W))
+    check(rc, "mq_dequant_fp8_block")
+    return out
+
+
 def gemm_f32_(A, sam, sak, B, sbk, sbn, Cm, M, N, K, alpha=1.0, beta=0.0, tri=0, ktrim=0):
     _dev(A, B, Cm)
     lib = _lib.load()

@@ -114,3 +114,48 @@ def get_relative_mse_error(q: Tensor, w: Tensor, H: Optional[Tensor] = None):
     if H is None:
         return delta.pow(2).mean() / w.pow(2).mean()
     return delta.mm(H).mul(delta).mean() / (w.mm(H).mul(w).mean() + 1e-6)
+
+
+FP8_GROUP_SIZE = 128  # src/quant_utils.py:16
+FP8_DTYPES = (torch.float8_e4m3fn, torch.float8_e4m3fnuz, torch.float8_e5m2, torch.float8_e5m2fnuz)  # :17
+
+
+def dequantize_weight_from_fp8(W: Tensor, s: Tensor) -> Tensor:
+    """src/quant_utils.py:267-284.  The reference receives W and s already cast to the target dtype and multiplies
+    them block by block.  An FP8 W (with s of the target dtype) takes the fused HIP kernel instead: same values,
+    one pass, no padded copies."""
+    if W.dtype == torch.float8_e4m3fn:
+        if s.dtype not in (torch.bfloat16, torch.float16):
+            raise TypeError("with an FP8 weight, s carries the target dtype: cast it to bfloat16 or float16")
+        return ops.dequant_fp8_block(W, s, s.dtype)
+    if W.dtype in FP8_DTYPES:
+        raise NotImplementedError(f"{W.dtype} checkpoints are not supported (DeepSeek ships float8_e4m3fn)")
+    g = FP8_GROUP_SIZE
+    d_out, d_in = W.shape
+    rows = torch.arange(d_out, device=W.device) // g
+    cols = torch.arange(d_in, device=W.device) // g
+    return W * s[rows][:, cols]
+
+
+def dequantize_state_dict(state_dict: dict, dtype: torch.dtype = torch.float16) -> None:
+    """src/quant_utils.py:287-298: every `<layer>.weight` that has a `<layer>.weight_scale_inv` is replaced by its
+    dequantized value in `dtype`, and the scale entry is dropped."""
+    for k in list(state_dict.keys()):
+        if k.endswith("scale_inv"):
+            layer_name, _ = k.rsplit(".", 1)
+            W = state_dict[f"{layer_name}.weight"]
+            s = state_dict[f"{layer_name}.weight_scale_inv"]
+            if W.dtype == torch.float8_e4m3fn and W.is_cuda:
+                # the reference rounds the scale to `dtype` first (s.to(dtype)); the kernel does the same
+                state_dict[f"{layer_name}.weight"] = ops.dequant_fp8_block(W, s.to(W.device), dtype)
+            else:
+                state_dict[f"{layer_name}.weight"] = dequantize_weight_from_fp8(W.to(dtype), s.to(dtype))
+            del state_dict[f"{layer_name}.weight_scale_inv"]
+
+
+def can_dequantize_from_fp8(state_dict: dict) -> bool:
+    """src/quant_utils.py:301-305."""
+    for k, v in state_dict.items():
+        if v.dtype in FP8_DTYPES and f"{k}_scale_inv" not in state_dict:
+            return False
+    return True

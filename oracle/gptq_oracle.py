@@ -27,6 +27,10 @@ pinned by closed forms / invariants / brute force in tests/test_oracle_*.py:
                               on the 4-bit grid keeps p = 1.  The bits of Triton's log/exp and the order of
                               its group sum decide near-ties between candidates: "parity unpinned" there.
 
+  dequantize_weight_from_fp8  known answers for e4m3fn bytes (0x38 = 1, 0x7e = 448, 0x01 = 2^-9, 0x7f = NaN) through
+                              torch's own fp8 cast; all 256 byte values against the format's definition; ragged
+                              shapes against a per-element loop
+
 Unpinnable by any means: torch.argsort tie order (unstable sort) and the exact
 bits of Triton's fma / division on a GPU.
 """
@@ -383,3 +387,30 @@ def pack_weight(weight: dict, bits: int, sym: bool, group_size: Optional[int] = 
     if not sym:
         out["weight_zero_point"] = weight["zero"]  # :73-74
     return out
+
+
+# ----------------------------------------------------------------------------------------------
+# checkpoint ingest -- src/quant_utils.py:267-298
+# ----------------------------------------------------------------------------------------------
+
+
+def dequantize_weight_from_fp8(W: Tensor, s: Tensor, g: int = 128) -> Tensor:
+    """src/quant_utils.py:267-284, statement by statement (pad, view as blocks, multiply, crop)."""
+    import math
+
+    import torch.nn.functional as F
+
+    d_out, d_in = W.shape
+    pad_out = math.ceil(d_out / g) * g - d_out
+    pad_in = math.ceil(d_in / g) * g - d_in
+    W = F.pad(W, (0, pad_in, 0, pad_out))
+    d_out_pad, d_in_pad = W.shape
+    W = W.view(d_out_pad // g, g, d_in_pad // g, g)
+    s = s.view(d_out_pad // g, 1, d_in_pad // g, 1)
+    W = (W * s).view(d_out_pad, d_in_pad)
+    return W[:d_out, :d_in]
+
+
+def dequantize_fp8_entry(W8: Tensor, scale_inv: Tensor, dtype: torch.dtype) -> Tensor:
+    """What dequantize_state_dict does to one (weight, weight_scale_inv) pair, src/quant_utils.py:292-296."""
+    return dequantize_weight_from_fp8(W8.to(dtype), scale_inv.to(dtype))

@@ -429,3 +429,26 @@ def test_mse_scale_search(dev, R, C, g, dtype):
     lg, lw = loss(got), loss(want)
     ok = ~torch.isnan(lw)  # fp16 rounds the 1e-12 scale of the all-zero group to 0: 0/0 there
     assert torch.all(lg[ok] <= lw[ok] * (1 + 1e-4) + 1e-30)
+
+
+# ---------------------------------------------------------------- FP8 checkpoint ingest (src/quant_utils.py:267-298)
+@pytest.mark.parametrize("R,C", [(256, 512), (130, 260), (7, 33), (2048, 7168)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp8_block_dequant_bit_exact(dev, R, C, dtype):
+    from moe_quant_amd import quant_utils
+
+    _say(f"fp8 dequant {R}x{C} {dtype}")
+    g = torch.Generator().manual_seed(R + C)
+    W8 = torch.randint(0, 256, (R, C), generator=g, dtype=torch.uint8)
+    W8[0, : min(C, 256)] = torch.arange(min(C, 256), dtype=torch.uint8)  # every byte value, NaNs included
+    W8 = W8.view(torch.float8_e4m3fn)
+    s = torch.rand((R + 127) // 128, (C + 127) // 128, generator=g) * 0.01 + 1e-4
+    want = O.dequantize_fp8_entry(W8, s, dtype)
+    got = ops.dequant_fp8_block(W8.to(dev), s.to(dev), dtype).cpu()
+    assert got.dtype == dtype
+    assert torch.equal(torch.nan_to_num(got.float(), nan=-77.0), torch.nan_to_num(want.float(), nan=-77.0))
+    sd = {"a.weight": W8.to(dev), "a.weight_scale_inv": s.to(dev), "b.weight": torch.ones(2, 2, device=dev)}
+    assert quant_utils.can_dequantize_from_fp8(sd)
+    quant_utils.dequantize_state_dict(sd, dtype)
+    assert set(sd) == {"a.weight", "b.weight"}
+    assert torch.equal(torch.nan_to_num(sd["a.weight"].float().cpu(), nan=-77.0), torch.nan_to_num(want.float(), nan=-77.0))

@@ -368,3 +368,35 @@ def test_mse_scale_special_cases():
         return (dq - x).abs().double().pow(2.4).sum(-1)
 
     assert torch.all(loss(got) <= loss(scale) * (1 + 1e-6))
+
+
+# ---------------------------------------------------------------- FP8 block dequantisation (src/quant_utils.py:267-298)
+def test_fp8_dequant_oracle_pins():
+    b = torch.arange(256, dtype=torch.uint8)
+    vals = b.view(torch.float8_e4m3fn).float()
+    # the format's definition: sign, 4-bit exponent (bias 7), 3-bit mantissa, no infinities, S.1111.111 = NaN
+    want = []
+    for x in range(256):
+        sgn, e, m = (-1.0 if x & 0x80 else 1.0), (x >> 3) & 15, x & 7
+        if e == 15 and m == 7:
+            want.append(float("nan"))
+        elif e == 0:
+            want.append(sgn * m * 2.0**-9)
+        else:
+            want.append(sgn * (1 + m / 8) * 2.0 ** (e - 7))
+    want = torch.tensor(want)
+    assert torch.equal(torch.nan_to_num(vals, nan=-77.0), torch.nan_to_num(want, nan=-77.0))
+    assert vals[0x38] == 1.0 and vals[0x7E] == 448.0 and vals[0x01] == 2.0**-9 and torch.isnan(vals[0x7F])
+    # ragged shape against a per-element loop
+    g = torch.Generator().manual_seed(5)
+    W8 = torch.randint(0, 256, (130, 260), generator=g, dtype=torch.uint8)
+    W8[W8 == 0x7F] = 0
+    W8[W8 == 0xFF] = 0
+    W8 = W8.view(torch.float8_e4m3fn)
+    s = torch.rand(2, 3, generator=g) * 0.01 + 1e-4
+    got = O.dequantize_fp8_entry(W8, s, torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and got.shape == (130, 260)
+    sb = s.to(torch.bfloat16)
+    for r, c in [(0, 0), (127, 127), (128, 128), (129, 259), (5, 200), (129, 0)]:
+        w = W8[r, c].to(torch.bfloat16)
+        assert got[r, c] == w * sb[r // 128, c // 128]
