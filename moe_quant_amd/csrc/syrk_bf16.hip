@@ -415,7 +415,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // lane its 8 tokens of a 32x32x16 operand; which tokens share a lane is irrelevant as long as both operands
 // use the same rule, and both are read by the same code.
 // Four stages are allocated: while stage s feeds the matrix cores, stages s+1..s+3 are in flight, tracked
-// with the vector-memory counter (8 loads per wavefront per stage), one barrier per stage.
+// with the vector-memory counter (32 loads per stage, shared evenly by the wavefronts), one barrier per stage.
 // =============================================================================================
 constexpr int KT3 = 32, NST3 = 4, CHUNK3 = 1024;
 constexpr int STAGE3 = (KT3 / 4) * 4 * CHUNK3;  // bytes
@@ -435,17 +435,17 @@ __device__ __forceinline__ void dma16(const void* sbase, unsigned lane_off, unsi
                : "memory", "m0");
 }
 
-// issues (or, for ragged stages, completes) the 8 chunk loads of this wavefront for the stage starting at token t0.
+// issues (or, for ragged stages, completes) the LPW chunk loads of this wavefront for the stage starting at token t0.
 // wave_u is the wavefront index as a scalar; lane_off = 2*(tau*ldx + 16*b + 8*half), the byte offset of this
 // lane's slot inside a chunk's source (4 token rows x 128 channels).
-template <bool FAST>
+template <bool FAST, int LPW>  // LPW: chunk loads per wavefront per stage (32 chunks / number of wavefronts)
 __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsigned lane_off, long ldx, int t0, int tend,
                                           int C, int m0, int n0, unsigned char* buf, unsigned lds_base, int wave_u,
                                           int lane) {
   const int b = lane >> 3, tau = (lane & 7) >> 1, half = lane & 1;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int ch = wave_u * 8 + i, q = ch >> 2, G = ch & 3;
+  for (int i = 0; i < LPW; ++i) {
+    const int ch = wave_u * LPW + i, q = ch >> 2, G = ch & 3;
     const int chan0 = ((G & 2) ? n0 : m0) + (G & 1) * 128;  // scalar
     if (FAST) {
       const long off = (long)(t0 + 4 * q) * ldx + chan0;  // scalar
@@ -462,14 +462,20 @@ __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsign
   }
 }
 
-// one 256x256 tile (or one token split of it); bid = linear workgroup index among ntri*splits
+// one 256x256 tile (or one token split of it); bid = linear workgroup index among ntri*splits.
+// NW = 4: four wavefronts of 128x128 (one per SIMD, all 512 registers).  NW = 8: eight of 128x64, two per SIMD:
+// while one waits for the address unit to take its direct loads the other keeps the matrix pipe busy.
+template <int NW>
 __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx,
                                               int n, int C, float alpha, float beta, int ntri, int splits,
                                               int tokens_per_split, float* __restrict__ ws, int bid,
                                               unsigned char* smem) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: LDS targets of the direct loads live in M0
-  const int wm = wave >> 1, wn = wave & 1;
+  constexpr int NJ = 16 / NW;     // 32-column blocks per wavefront: 4 (128 columns) or 2 (64 columns)
+  constexpr int WCOLS = NW / 2;   // wavefronts side by side along the columns
+  constexpr int LPW = 32 / NW;    // direct loads per wavefront per stage
+  const int wm = wave / WCOLS, wn = wave % WCOLS;
   const int L = xcd_remap(bid, ntri * splits);
   const int split = L / ntri;
   int tm, tn;
@@ -488,11 +494,11 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
       (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem);
   const unsigned lane_off = 2u * (unsigned)(((lane & 7) >> 1) * ldx + 16 * (lane >> 3) + 8 * (lane & 1));
 
-  floatx16 acc[4][4];
+  floatx16 acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -501,8 +507,8 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
     const int t0_ = tbeg + (st)*KT3;                                                              \
     unsigned char* buf_ = smem + ((st) % NST3) * STAGE3;                                          \
     const unsigned lds_ = smem_lds + (unsigned)(((st) % NST3) * STAGE3);                          \
-    if (interior && t0_ + KT3 <= tend) dma_stage<true>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);  \
-    else dma_stage<false>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);        \
+    if (interior && t0_ + KT3 <= tend) dma_stage<true, LPW>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);  \
+    else dma_stage<false, LPW>(X, lane_off, ldx, t0_, tend, C, m0, n0, buf_, lds_, wave, lane);        \
   } while (0)
 
 #pragma unroll
@@ -512,7 +518,8 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
   // fragment addressing: 16-lane group g16 = lane/16 -> channel block parity g16&1, token half g16>>1
   const int g16 = lane >> 4, s16 = lane & 15;
   const int a_off = wm * CHUNK3 + (g16 & 1) * 128 + s16 * 8;        // + i*256 (block pair i) + quad*4*CHUNK3
-  const int b_off = (2 + wn) * CHUNK3 + (g16 & 1) * 128 + s16 * 8;  // + j*256
+  const int co = wn * NJ * 32;  // first column of this wavefront inside the column tile
+  const int b_off = (2 + co / 128) * CHUNK3 + ((co % 128) / 16 + (g16 & 1)) * 128 + s16 * 8;  // + j*256
   const int hq = g16 >> 1;
 
   for (int kt = 0; kt < nk; ++kt) {
@@ -520,9 +527,11 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
     const int ahead = min(nk, kt + NST3 - 1) - (kt + 1);
     // (lgkmcnt(0) as well: LDS writes of a ragged stage must have landed before the barrier lets others read)
     asm volatile("" ::: "memory");
-    if (ahead >= 2) __builtin_amdgcn_s_waitcnt(0x4070);       // vmcnt(16) lgkmcnt(0)
-    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
-    else __builtin_amdgcn_s_waitcnt(0x0070);                  // vmcnt(0) lgkmcnt(0)
+    // s_waitcnt immediates: vmcnt in bits 3:0 and 15:14, expcnt 6:4 left at its maximum, lgkmcnt(0) in 11:8
+    constexpr int W2 = 0x0070 | ((2 * LPW) & 15) | (((2 * LPW) >> 4) << 14), W1 = 0x0070 | LPW;
+    if (ahead >= 2) __builtin_amdgcn_s_waitcnt(W2);       // vmcnt(2*LPW) lgkmcnt(0)
+    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(W1);  // vmcnt(LPW) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);              // vmcnt(0) lgkmcnt(0)
     // a bare barrier: __syncthreads() carries a fence that makes the compiler drain every direct load in flight.
     // The empty asm statements keep the compiler from moving LDS accesses across it.
     __builtin_amdgcn_s_barrier();
@@ -531,28 +540,28 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
     const unsigned char* stg = smem + (kt % NST3) * STAGE3;
 #pragma unroll
     for (int kk = 0; kk < KT3 / 16; ++kk) {
-      short4v fa[4][2], fb[4][2];
+      short4v fa[4][2], fb[NJ][2];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
         const int quad = 4 * kk + 2 * r + hq;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 4; ++i)
           fa[i][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
               (short4v __attribute__((address_space(3)))*)(stg + quad * 4 * CHUNK3 + a_off + i * 256));
-          fb[i][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (short4v __attribute__((address_space(3)))*)(stg + quad * 4 * CHUNK3 + b_off + i * 256));
-        }
-      }
-      bf16x8 va[4], vb[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        va[i] = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, 6, 7);
-        vb[i] = __builtin_shufflevector(fb[i][0], fb[i][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int j = 0; j < NJ; ++j)
+          fb[j][r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(stg + quad * 4 * CHUNK3 + b_off + j * 256));
       }
+      bf16x8 va[4], vb[NJ];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) va[i] = __builtin_shufflevector(fa[i][0], fa[i][1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) vb[j] = __builtin_shufflevector(fb[j][0], fb[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8n, va[i]),
                                                               __builtin_bit_cast(bf16x8n, vb[j]), acc[i][j], 0, 0, 0);
     }
@@ -565,8 +574,8 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int c = wn * 128 + j * 32 + lr;
+    for (int j = 0; j < NJ; ++j) {
+      const int c = co + j * 32 + lr;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
@@ -586,7 +595,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
     int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  syrk_dma_tile(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+  syrk_dma_tile<4>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+}
+
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_bf16_dma8_kernel(
+    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
+    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  syrk_dma_tile<8>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
 }
 
 // Several independent accumulations (one Hessian each, same C) in one launch: blockIdx.y picks the problem.
@@ -600,12 +616,12 @@ struct SyrkGroupTable {
   int n[SYRK_MAX_GROUP];
   float alpha[SYRK_MAX_GROUP], beta[SYRK_MAX_GROUP];
 };
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_grouped_kernel(
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_bf16_dma_grouped_kernel(
     SyrkGroupTable t, int C, int ntri) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int z = blockIdx.y;
   const int tps = (t.n[z] + KT3 - 1) / KT3 * KT3;
-  syrk_dma_tile(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
+  syrk_dma_tile<8>(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
                 smem);
 }
 
@@ -741,10 +757,16 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
                                 (int)BIG_SMEM);
       (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)DMA_SMEM);
+      (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)DMA_SMEM);
       use_dma = getenv("MQ_SYRK_OLD") == nullptr;
       big_attr = true;
     }
-    if (use_dma)
+    static const int dma_waves = getenv("MQ_SYRK_W4") ? 4 : 8;  // the one-wavefront-per-SIMD kernel stays for comparison
+    if (use_dma && dma_waves == 8)
+      hipLaunchKernelGGL(syrk_bf16_dma8_kernel, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
+                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    else if (use_dma)
       hipLaunchKernelGGL(syrk_bf16_dma_kernel, dim3(ntri * splits), dim3(256), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
                          ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
     else
@@ -831,7 +853,7 @@ extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const l
       t.alpha[i] = alpha[g];
       t.beta[i] = beta[g];
     }
-    hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel, dim3(ntri, cnt), dim3(256), DMA_SMEM, st, t, C, ntri);
+    hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel, dim3(ntri, cnt), dim3(512), DMA_SMEM, st, t, C, ntri);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     if (mirror)
