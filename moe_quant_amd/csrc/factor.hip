@@ -27,75 +27,237 @@ namespace {
 
 constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
-constexpr int LDM = 131;   // LDS row pitch (odd: lane-per-row accesses hit 32 distinct banks)
+constexpr int LDM = 132;   // LDS row pitch: rows 16-byte aligned, consecutive rows 4 banks apart (8 rows span the 32 banks)
+constexpr int SOFF = 4;    // column shift of the S triangle inside a row (keeps both triangles 16-byte aligned)
 static int INV_KC = 4;  // the first inverse product is cut into K chunks of 4 blocks (512), one workgroup each
 
 // ---------------------------------------------------------------------------------------------
 // Diagonal block: S (128x128, upper valid) -> R^-1 where S = R R^T, R upper.
 //
 // One LDS array holds two triangular matrices side by side: the upper triangle S(i,k), k >= i, at
-// column k+1, and below it Xt(c,k) = X[k][c], k <= c, at column k, where X accumulates R^-1.
-// Stacking M = [S; Xt] makes the inverse fall out of the factorisation: every elimination step that
-// scales column j of S by 1/R_jj and subtracts its outer product from the columns to its left does,
-// applied unchanged to the rows of Xt (initialised to the identity), exactly the right-looking update
-// of the triangular inverse.  Nothing extra is computed for the inverse except more rows.
+// column k+4, and below it Xt(c,k) = X[k][c], k <= c, at column k, where X accumulates R^-1 (columns
+// i+1..i+3 of row i belong to neither).  Stacking M = [S; Xt] makes the inverse fall out of the
+// factorisation: every elimination step that scales column j of S by 1/R_jj and subtracts its outer product
+// from the columns to its left does, applied unchanged to the rows of Xt (initialised to the identity),
+// exactly the right-looking update of the triangular inverse.  Nothing extra is computed for the inverse
+// except more rows.
 //
 // Sub-blocks of 32: the 32x32 diagonal sub-block is eliminated by one wavefront with a row per lane in
 // registers -- lanes 0-31 carry S rows, lanes 32-63 the matching Xt rows, same instructions -- and the
 // off-diagonal work (column scaling by the sub-block inverse, outer-product updates) runs as 32x32x32
 // products on the fp32 matrix cores, one product per wavefront at a time.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float& Sv(float* buf, int i, int k) { return buf[i * LDM + k + 1]; }
+__device__ __forceinline__ float& Sv(float* buf, int i, int k) { return buf[i * LDM + k + SOFF]; }
 __device__ __forceinline__ float& Xv(float* buf, int c, int k) { return buf[c * LDM + k]; }
 
 __device__ __forceinline__ float bcast_lane(float v, int lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+
+// acc -= rep[lane N of this lane's row of 16 lanes] * v, one instruction (a DPP row broadcast feeds the multiplier)
+template <int N, bool FIRST>
+__device__ __forceinline__ void fmac_rowbcast(float& acc, float rep, float v) {
+  // FIRST: two wait states, required between the instruction that wrote rep and a DPP read of it; the
+  // compiler cannot see that this statement is a DPP instruction, so the first of a run carries them itself
+  if (FIRST)
+    asm("s_nop 1\n\tv_fmac_f32_dpp %0, -%1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(rep), "v"(v), "n"(N));
+  else
+    asm("v_fmac_f32_dpp %0, -%1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(rep), "v"(v), "n"(N));
+}
+
+// columns K..0 of the rank-one update of the step before: reg[k] -= v_k * v; nearest column first, it holds the
+// next pivot
+template <int K, int TOP>
+struct RankOne {
+  static __device__ __forceinline__ void run(float (&reg)[SB], float lo, float hi, float v) {
+    if constexpr (K >= 0) {
+      fmac_rowbcast<(K & 15), K == TOP>(reg[K], K < 16 ? lo : hi, v);
+      RankOne<K - 1, TOP>::run(reg, lo, hi, v);
+    }
+  }
+};
+
+// One elimination step on column J of the 32x32 sub-block held one row per lane in reg[].
+// The rank-one update of step J needs v_k (the value lane k holds) as a multiplier common to all lanes, for
+// every column k < J.  The 32 multipliers are replicated into every row of 16 lanes (lo: v_0..v_15, hi:
+// v_16..v_31; two lane swaps) and each column then costs one multiply-add whose multiplier operand is a DPP row
+// broadcast; those updates are applied one step late (vprev/lo/hi carry step J+1's vector and multipliers into
+// step J), which takes the lane swaps off the dependence chain from pivot to pivot.
+// The chain itself runs on values every lane holds alike, so it needs no cross-lane read at all: with
+// s = S(J-1,J) and e = S(J-1,J-1), both read across lanes before the pivot's reciprocal root y is known, the
+// next pivot is e - (s*y)^2: rsq, multiply, multiply-add per step.  Only the next pivot column is updated at once.
+// A pivot that is not positive turns everything after it into NaN; the caller checks the diagonal afterwards.
 template <int J>
 struct ElimStep {
-  // one elimination step on column J of the 32x32 sub-block held one row per lane in reg[]
-  static __device__ __forceinline__ void run(float (&reg)[SB], int gidx, int& bad) {
-    float d = bcast_lane(reg[J], J);
-    const bool neg = !(d > 0.f);  // also catches NaN; selects, not branches: one basic block per sub-block
-    bad = (neg && bad == 0) ? (gidx + J + 1) : bad;
-    d = neg ? 1.f : d;
-    float y = __frsqrt_rn(d);
-    y = y * (1.5f - 0.5f * d * y * y);  // one Newton step: 1/sqrt(d) to fp32 accuracy
+  static __device__ __forceinline__ void run(float (&reg)[SB], float dv, float vprev, float lo, float hi) {
+    if constexpr (J + 1 < SB) RankOne<J - 1, J - 1>::run(reg, lo, hi, vprev);  // step J+1's updates of the columns k < J
+    const float y = __frsqrt_rn(dv);
+    float dnext = 0.f;
+    float c = 0.f;
+    if constexpr (J >= 1) {
+      c = bcast_lane(reg[J], J - 1) * y;
+      dnext = fmaf(-c, c, bcast_lane(reg[J - 1], J - 1));
+    }
     const float v = reg[J] * y;
     reg[J] = v;
-    // nearest column first: the next step's pivot lives in reg[J-1], so its chain can start while the
-    // remaining updates of this step are still issuing
-#pragma unroll
-    for (int k = J - 1; k >= 0; --k) reg[k] = fmaf(-bcast_lane(v, k), v, reg[k]);
-    ElimStep<J - 1>::run(reg, gidx, bad);
+    if constexpr (J >= 1) reg[J - 1] = fmaf(-c, v, reg[J - 1]);
+    float nlo = 0.f, nhi = 0.f;
+    if constexpr (J >= 2) {
+      const unsigned vu = __float_as_uint(v);
+      const uintx2 t = __builtin_amdgcn_permlane32_swap(vu, vu, false, false);      // t[0]: lanes 0..31 twice
+      const uintx2 u = __builtin_amdgcn_permlane16_swap(t[0], t[0], false, false);  // lanes 0..15 / 16..31 four times
+      nlo = __uint_as_float(u[0]);
+      nhi = __uint_as_float(u[1]);
+    }
+    // the instruction scheduler must not carry work across steps: left alone it postpones every column's updates
+    // to the step that needs the column, which keeps all multipliers of all steps alive and puts them on the chain
+    __builtin_amdgcn_sched_barrier(0);
+    ElimStep<J - 1>::run(reg, dnext, v, nlo, nhi);
   }
 };
 template <>
 struct ElimStep<-1> {
-  static __device__ __forceinline__ void run(float (&)[SB], int, int&) {}
+  static __device__ __forceinline__ void run(float (&)[SB], float, float, float, float) {}
 };
 
-// acc (32x32, MFMA layout) (+)= sum_k a(m,k) * b(k,n); a/b fetch one element for this lane
-template <typename FA, typename FB>
-__device__ __forceinline__ void mm32(floatx16& acc, FA a, FB b, int lane) {
-  const int x = lane & 31, kk = lane >> 5;
-  float av[16], bv[16];
+// 16 consecutive floats (16-byte aligned) from LDS
+__device__ __forceinline__ void ld16(const float* p, float (&v)[16]) {
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    av[t] = a(x, 2 * t + kk);
-    bv[t] = b(2 * t + kk, x);
+  for (int q = 0; q < 4; ++q) {
+    const floatx4 t = *reinterpret_cast<const floatx4*>(p + 4 * q);
+    v[4 * q + 0] = t[0];
+    v[4 * q + 1] = t[1];
+    v[4 * q + 2] = t[2];
+    v[4 * q + 3] = t[3];
   }
-#pragma unroll
-  for (int t = 0; t < 16; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], bv[t], acc, 0, 0, 0);
 }
 
-// buf: LDS, NB*LDM floats.  blk: global 128x128 block (row pitch ld).  gidx0: global index of its first row.
-// preloaded: the caller already filled Sv (upper) and zeroed Xv (strictly lower) and synchronised.
-// blk rows must be 16-byte aligned (ld % 4 == 0).
+// 32x32x32 products on LDS tiles (row pitch LDM, tile origins 16-byte aligned), one wavefront each.
+// Lane (x = lane%32, h = lane/32) supplies k = 16h..16h+15 of row x of both operands -- 64 contiguous bytes --
+// and the product is formed transposed (operands swapped), so that the lane ends up with row x of C as four
+// runs of four consecutive columns: C too moves 16 bytes at a time.
+//   tile_update:  C(m,n) -= sum_k A(m,k) * B(n,k)        A_LOWER: A(m,k) counts only for k <= m
+template <bool A_LOWER>
+__device__ __forceinline__ void tile_update(float* c, const float* a, const float* b, int lane) {
+  int x = lane & 31;
+  asm volatile("" : "+v"(x));  // keeps the masks below from being hoisted out of the caller's loops
+  const int h = lane >> 5;
+  float av[16], bv[16];
+  ld16(a + x * LDM + 16 * h, av);
+  ld16(b + x * LDM + 16 * h, bv);
+  floatx16 acc;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const floatx4 t = *reinterpret_cast<const floatx4*>(c + x * LDM + 8 * g + 4 * h);
+    acc[4 * g + 0] = t[0];
+    acc[4 * g + 1] = t[1];
+    acc[4 * g + 2] = t[2];
+    acc[4 * g + 3] = t[3];
+  }
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    float an = -av[t];
+    if (A_LOWER) an = (16 * h + t <= x) ? an : 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[t], an, acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    floatx4 t;
+    t[0] = acc[4 * g + 0];
+    t[1] = acc[4 * g + 1];
+    t[2] = acc[4 * g + 2];
+    t[3] = acc[4 * g + 3];
+    *reinterpret_cast<floatx4*>(c + x * LDM + 8 * g + 4 * h) = t;
+  }
+}
+//   tile_scale:  A(m,n) <- sum_{k >= n} A(m,k) * Xi(k,n), Xi = the lower-triangular Xt tile of the sub-block (in place)
+//   tr != nullptr: the result is final (an Xt tile of the inverse); its transpose is also stored at tr
+template <bool COPY_T>
+__device__ __forceinline__ void tile_scale(float* a, const float* xi, float* tr, int lane) {
+  int x = lane & 31;
+  asm volatile("" : "+v"(x));  // keeps the masks below from being hoisted out of the caller's loops
+  const int h = lane >> 5;
+  float av[16], bv[16];
+  ld16(a + x * LDM + 16 * h, av);
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const float e = xi[(16 * h + t) * LDM + x];
+    bv[t] = (16 * h + t >= x) ? e : 0.f;
+  }
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[t], av[t], acc, 0, 0, 0);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    floatx4 t;
+    t[0] = acc[4 * g + 0];
+    t[1] = acc[4 * g + 1];
+    t[2] = acc[4 * g + 2];
+    t[3] = acc[4 * g + 3];
+    *reinterpret_cast<floatx4*>(a + x * LDM + 8 * g + 4 * h) = t;
+  }
+  if (COPY_T) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) tr[(8 * (v >> 2) + 4 * h + (v & 3)) * LDM + x] = acc[v];
+  }
+}
+
+constexpr int LDI = 36;  // row pitch of the 32x32 identity kept behind the matrix (same bank spread as LDM)
+
+// one wavefront: eliminate the diagonal sub-block at offset o; leaves the sub-block of the inverse in Xt and,
+// transposed, in the S triangle
+__device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, int gidx, int* info) {
+  float reg[SB];
+  const int li = lane & 31;
+  const bool up = lane >= 32;
+  float* row = buf + (o + li) * LDM + o;
+  // S rows start from S (what a row holds left of its diagonal is other data: it stays in that lane's registers,
+  // no other lane ever reads it), Xt rows from the identity
+  const float* src = up ? buf + NB * LDM + li * LDI : row + SOFF;
+#pragma unroll
+  for (int q = 0; q < SB / 4; ++q) {
+    const floatx4 t = *reinterpret_cast<const floatx4*>(src + 4 * q);
+    reg[4 * q + 0] = t[0];
+    reg[4 * q + 1] = t[1];
+    reg[4 * q + 2] = t[2];
+    reg[4 * q + 3] = t[3];
+  }
+  ElimStep<SB - 1>::run(reg, bcast_lane(reg[SB - 1], SB - 1), 0.f, 0.f, 0.f);
+  // The S rows are not written back: R itself is never read again.  The Xt rows hold the sub-block of the inverse.
+  // First its transpose goes into the S triangle, where the finished inverse is collected row-major for the
+  // write to memory (the zeros right of a row's diagonal land left of another row's: Xt or unused columns);
+  // then the rows themselves, in place, for the products that follow (the quad that straddles the diagonal
+  // spills zeros into the unused columns li+1..li+3 only).
+  if (up) {
+#pragma unroll
+    for (int k = 0; k < SB; ++k) Sv(buf, o + k, o + li) = reg[k];
+#pragma unroll
+    for (int q = 0; q < SB / 4; ++q) {
+      const floatx4 t = {reg[4 * q], reg[4 * q + 1], reg[4 * q + 2], reg[4 * q + 3]};
+      if (q <= (li >> 2)) *reinterpret_cast<floatx4*>(row + 4 * q) = t;
+    }
+  }
+  // 1/R_jj sits on the diagonal just written: positive and finite unless pivot j or one before it failed.
+  // Reported: the first failure in walking order, i.e. the highest column.
+  const float dg = up ? Sv(buf, o + li, o + li) : 1.f;
+  const unsigned long long fail = __ballot(!(dg > 0.f && dg < 3.0e38f));
+  if (fail != 0 && lane == 0) atomicCAS(info, 0, gidx + 32 - __builtin_clzll(fail));
+}
+
+// buf: LDS, NB*LDM floats followed by a 32 x LDI identity.  blk: global 128x128 block (row pitch ld).
+// gidx0: global index of its first row.  preloaded: the caller already filled Sv (upper) and zeroed the 32x32 Xt
+// tiles below the diagonal ones (a barrier here orders those writes).  blk rows must be 16-byte aligned.
 __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info,
                                                   bool preloaded) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int idx = tid; idx < SB * LDI; idx += 256) buf[NB * LDM + idx] = (idx / LDI == idx % LDI) ? 1.f : 0.f;
+  if (preloaded) __syncthreads();
   if (!preloaded) {
     float4 v[16];
 #pragma unroll
@@ -118,90 +280,53 @@ __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long l
 
   for (int J = NB / SB - 1; J >= 0; --J) {
     const int o = J * SB;
-    if (wave == 0) {
-      float reg[SB];
-      const int li = lane & 31;
-      const bool up = lane >= 32;
-#pragma unroll
-      for (int k = 0; k < SB; ++k) reg[k] = up ? (k == li ? 1.f : 0.f) : (k >= li ? Sv(buf, o + li, o + k) : 0.f);
-      int bad = 0;
-      ElimStep<SB - 1>::run(reg, gidx0 + o, bad);
-      if (bad != 0 && lane == 0) atomicCAS(info, 0, bad);
-#pragma unroll
-      for (int k = 0; k < SB; ++k) {
-        if (!up && k >= li) Sv(buf, o + li, o + k) = reg[k];
-        if (up && k <= li) Xv(buf, o + li, o + k) = reg[k];
-      }
-    }
-    __syncthreads();
-    // ---- column block J of M times the sub-block inverse: V = M(:,J) * Xinv^T, Xinv[n][k] = Xt(o+k... ) masked
-    {
-      const int ntask = 3;  // J row blocks of S above the diagonal + (3-J) row blocks of Xt below it
-      for (int t = wave; t < ntask; t += 4) {
-        const bool is_s = t < J;
-        const int rb = is_s ? t : (t + 1);  // S row block I=t, or Xt row block Cb=t+1 (> J)
-        const int ro = rb * SB;
-        floatx16 acc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-        auto bfn = [&](int k, int n) { return (k >= n) ? Xv(buf, o + k, o + n) : 0.f; };  // Xinv[n][k]
-        if (is_s) mm32(acc, [&](int m, int k) { return Sv(buf, ro + m, o + k); }, bfn, lane);
-        else mm32(acc, [&](int m, int k) { return Xv(buf, ro + m, o + k); }, bfn, lane);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
-          if (is_s) Sv(buf, ro + m, o + n) = acc[v];
-          else Xv(buf, ro + m, o + n) = acc[v];
-        }
-      }
-    }
-    __syncthreads();
-    // ---- outer-product updates of the column blocks K < J:  M(rb,K) -= V(rb) * R(K,J)^T
-    {
-      // tasks enumerated as (K, rb): for each K < J the S row blocks I <= K, then the Xt row blocks Cb >= J
-      const int per_k_x = NB / SB - J;
+    // ---- phase: outer-product updates owed by column block Jp = J+1:  M(rb,K) -= V(rb) * R(K,Jp)^T for K <= J,
+    //      over the S row blocks rb <= K and the Xt row blocks rb >= Jp.  Wavefront 0 takes the one tile the
+    //      next elimination needs, S(J,J), and goes straight on to eliminate it; the others share the rest.
+    if (J + 1 < NB / SB) {
+      const int Jp = J + 1, op = Jp * SB;
+      const int per_k_x = NB / SB - Jp;
       int t = 0;
-      for (int K = 0; K < J; ++K) {
+      for (int K = J; K >= 0; --K) {
         const int cnt = (K + 1) + per_k_x;
-        for (int q = 0; q < cnt; ++q, ++t) {
-          if ((t & 3) != wave) continue;
+        for (int q = cnt - 1; q >= 0; --q) {
           const bool is_s = q <= K;
-          const int rb = is_s ? q : (J + (q - K - 1));
+          const int rb = is_s ? q : (Jp + (q - K - 1));
+          const bool critical = is_s && K == J && rb == J;
+          if (critical ? (wave != 0) : (wave == 0 || (t++ % 3) != wave - 1)) continue;
           const int ro = rb * SB, ko = K * SB;
-          floatx16 acc;
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
-            acc[v] = is_s ? Sv(buf, ro + m, ko + n) : Xv(buf, ro + m, ko + n);
-          }
-          auto bfn = [&](int k, int n) { return Sv(buf, ko + n, o + k); };  // R(K,J)[n][k]
-          if (is_s) {
-            mm32(acc, [&](int m, int k) { return -Sv(buf, ro + m, o + k); }, bfn, lane);
-          } else if (rb == J) {  // V is the sub-block inverse itself; only its lower triangle is Xt data
-            mm32(acc, [&](int m, int k) { return (k <= m) ? -Xv(buf, ro + m, o + k) : 0.f; }, bfn, lane);
-          } else {
-            mm32(acc, [&](int m, int k) { return -Xv(buf, ro + m, o + k); }, bfn, lane);
-          }
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int m = 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), n = lane & 31;
-            if (is_s) Sv(buf, ro + m, ko + n) = acc[v];
-            else Xv(buf, ro + m, ko + n) = acc[v];
-          }
+          const int sh = is_s ? SOFF : 0;
+          float* c = buf + ro * LDM + ko + sh;
+          const float* a = buf + ro * LDM + op + sh;
+          const float* b = buf + ko * LDM + op + SOFF;  // R(K,Jp), rows n, columns k
+          if (!is_s && rb == Jp) tile_update<true>(c, a, b, lane);  // V is the sub-block inverse: lower triangle only
+          else tile_update<false>(c, a, b, lane);
         }
       }
+    }
+    // ---- phase: elimination of the diagonal sub-block
+    if (wave == 0) eliminate_subblock(buf, o, lane, gidx0 + o, info);
+    __syncthreads();
+    // ---- phase: column block J of M times the sub-block inverse: J row blocks of S above the diagonal,
+    //      3-J row blocks of Xt below it (those are final: also copied, transposed, into the S triangle)
+    for (int t = wave; t < 3; t += 4) {
+      const bool is_s = t < J;
+      const int ro = (is_s ? t : t + 1) * SB;
+      if (is_s) tile_scale<false>(buf + ro * LDM + o + SOFF, buf + o * LDM + o, nullptr, lane);
+      else tile_scale<true>(buf + ro * LDM + o, buf + o * LDM + o, buf + o * LDM + ro + SOFF, lane);
     }
     __syncthreads();
   }
-  // R^-1[r][c] = Xt(c, r) for r <= c, zero below the diagonal
+  // ---- phase: the S triangle now holds R^-1 row-major; written row by row, zero below the diagonal
 #pragma unroll 4
   for (int it = 0; it < 16; ++it) {
     const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+    const floatx4 t = *reinterpret_cast<const floatx4*>(buf + r * LDM + SOFF + c);
     float4 o4;
-    o4.x = (r <= c + 0) ? Xv(buf, c + 0, r) : 0.f;
-    o4.y = (r <= c + 1) ? Xv(buf, c + 1, r) : 0.f;
-    o4.z = (r <= c + 2) ? Xv(buf, c + 2, r) : 0.f;
-    o4.w = (r <= c + 3) ? Xv(buf, c + 3, r) : 0.f;
+    o4.x = (r <= c + 0) ? t[0] : 0.f;
+    o4.y = (r <= c + 1) ? t[1] : 0.f;
+    o4.z = (r <= c + 2) ? t[2] : 0.f;
+    o4.w = (r <= c + 3) ? t[3] : 0.f;
     *reinterpret_cast<float4*>(blk + (long)r * ld + c) = o4;
   }
 }
@@ -253,14 +378,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
   const int bid = blockIdx.x;
   if (bid == 0) {
     const int t = i1 / NB - 1;  // last tile of the column-major upper-triangle order
-    tile_body<true, true, true>(g, t, t, 0, buf, 1, 1, [&](int r, int c, float v) {
-      if (c >= r) Sv(buf, r, c) = v;
-    });
-    for (int idx = threadIdx.x; idx < NB * NB; idx += 256) {
-      const int r = idx >> 7, c = idx & 127;
-      if (c < r) Xv(buf, r, c) = 0.f;
-    }
+    // the whole tile goes to the S position: what lies left of a row's diagonal lands in that row's Xt or unused
+    // columns, and the Xt part is cleared next
+    tile_body<true, true, true>(g, t, t, 0, buf, 1, 1, [&](int r, int c, float v) { Sv(buf, r, c) = v; });
     __syncthreads();
+    // Xt starts at zero in its 32x32 tiles below the diagonal ones (those are written whole by the elimination)
+    for (int idx = threadIdx.x; idx < (NB - SB) * (NB / 4); idx += 256) {
+      const int r = SB + idx / (NB / 4), q = idx % (NB / 4);
+      if (q < (r / SB) * (SB / 4)) *reinterpret_cast<floatx4*>(buf + r * LDM + 4 * q) = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
     diag_block_invert(buf, A + (long)(i1 - NB) * ld + (i1 - NB), ld, i1 - NB, info, true);
   } else if (bid <= inv_tiles) {
     inv_first_tile(ginv, kc, bid - 1, buf);
@@ -305,7 +431,7 @@ __global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C
   }
 }
 
-constexpr size_t DIAG_SMEM = (size_t)(NB * LDM) * sizeof(float);
+constexpr size_t DIAG_SMEM = (size_t)(NB * LDM + SB * LDI) * sizeof(float);
 constexpr size_t FUSED_SMEM = DIAG_SMEM > gemmf32::SMEM_BYTES ? DIAG_SMEM : gemmf32::SMEM_BYTES;
 
 }  // namespace
