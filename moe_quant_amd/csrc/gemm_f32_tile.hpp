@@ -180,7 +180,22 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
   } while (0)
   const int nk = (ke - kb + BK - 1) / BK;
   if (nk > 0) MQ_GEMM_FETCH(kb);
-  if (beta != 0.f) {
+  // Interior tiles that go to memory move C sixteen bytes at a time, row-wise (a wavefront covers two rows of 512
+  // bytes per instruction): the old tile is fetched that way here, and the result is turned from the MFMA layout
+  // into that layout through LDS once the operand stages are no longer needed.
+  constexpr bool ROWWISE_C = FAST && !LDS_OUT;
+  constexpr int LDC_S = BN + 4;  // LDS row pitch of the result tile
+  static_assert(BM * LDC_S <= 4 * STAGE, "result tile must fit in the operand stages");
+  floatx4 cold4[ROWWISE_C ? 16 : 1];
+  if (ROWWISE_C) {
+    if (beta != 0.f) {
+#pragma unroll
+      for (int it = 0; it < 16; ++it) {
+        const int idx = tid + it * 256;
+        cold4[it] = *reinterpret_cast<const floatx4*>(C + (long)(m0 + (idx >> 5)) * g.ldc + n0 + ((idx & 31) << 2));
+      }
+    }
+  } else if (beta != 0.f) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -224,6 +239,31 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
     __syncthreads();
   }
 
+  if (ROWWISE_C) {
+    float* cs = smem;  // the loop's last barrier has passed: no wavefront reads operands any more
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          cs[(wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3)) * LDC_S + wn * 64 + j * 32 + lr] = acc[i][j][v];
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+      const floatx4 a4 = *reinterpret_cast<const floatx4*>(cs + r * LDC_S + c);
+      floatx4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float x = alpha * a4[e];
+        if (beta != 0.f) x = fmaf(beta, cold4[it][e], x);
+        o[e] = x;
+      }
+      *reinterpret_cast<floatx4*>(C + (long)(m0 + r) * g.ldc + n0 + c) = o;
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -261,7 +301,8 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   int kb = 0, ke = g.K;
   if (g.ktrim == 1) ke = min(g.K, m0 + BM);
   if (g.ktrim == 2) kb = m0;
-  const bool interior = vecA && vecB && m0 + BM <= g.M && n0 + BN <= g.N && ((ke - kb) % BK == 0);
+  const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0);  // C moves 16 bytes at a time
+  const bool interior = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N && ((ke - kb) % BK == 0);
   if (interior) tile_core<A_KC, B_KC, true, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
   else tile_core<A_KC, B_KC, false, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
 }

@@ -62,12 +62,46 @@ constexpr int UT_FLOATS = 36 * 256;
 
 typedef const int __attribute__((address_space(4))) * cint_p;  // constant address space: scalar loads
 
+// x[t] += sum_J U[j0+J, k0+t] * e[J] for the 16 columns k0.. and the 16 errors of columns j0.. (ascending J, one fma
+// each).  The multipliers are the same for every lane: read from LDS with all lanes on one address (a broadcast,
+// four values per read), four rows of U at a time, one group ahead of the FMAs.  (Scalar loads of U from memory,
+// which would keep the multipliers out of the vector registers, measured slower: they wait on L2.)
+__device__ __forceinline__ void fold16(const float* ut, const float (&e)[MB], int j0, int k0, float (&x)[MB]) {
+  float4 ug[2][4][MB / 4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+    for (int t4 = 0; t4 < MB / 4; ++t4) ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(j0 + jj, k0 + 4 * t4)]);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    if (g < 3) {
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+        for (int t4 = 0; t4 < MB / 4; ++t4)
+          ug[(g + 1) & 1][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(j0 + 4 * (g + 1) + jj, k0 + 4 * t4)]);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const float ej = e[4 * g + jj];
+#pragma unroll
+      for (int t4 = 0; t4 < MB / 4; ++t4) {
+        const float4 u = ug[g & 1][jj][t4];
+        x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
+        x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
+        x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
+        x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
+      }
+    }
+  }
+}
+
 // One workgroup (four wavefronts) owns 64 rows; lane l of every wavefront is row l.  The 128-column
 // block of those rows sits in LDS ([column][lane], so every access is conflict-free) next to the
 // 128x128 block of U.  16 columns at a time move to the registers of wavefront 0 for the strictly
-// sequential part; their 16 errors are published in LDS and all four wavefronts fold them into the rest
-// of the block, each taking every fourth pass of 16 columns.  The multipliers U[j,k] are the same for
-// every lane: they are read from LDS with all lanes on one address (a broadcast, four values per read).
+// sequential part; their 16 errors are published in LDS.  While wavefront 0 walks the next 16 columns (after
+// folding those errors into them itself), the other three wavefronts fold them into the rest of the block, each
+// taking every third pass of 16 columns.
 // For every weight the updates are applied in ascending j with one fma each, exactly the order of the
 // sequential reference.
 //
@@ -85,7 +119,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   }
   float* tile = reinterpret_cast<float*>(smem);  // [B][WSTRIDE]
   float* ut = tile + B * WSTRIDE;                // packed upper micro-blocks of the U block
-  float* esh = ut + UT_FLOATS;                   // [MB][WSTRIDE] errors of the current micro-block
+  float* esh = ut + UT_FLOATS;                   // [2][MB][WSTRIDE] errors of the current and the previous micro-block
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r0 = blockIdx.x * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
@@ -107,19 +141,27 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
     // straight from memory in MFMA layout (lane = column, the two k of an instruction in the two lane halves),
     // every load issued before the first product.
     float* es = ut;  // [nbprev][64]
-    for (int idx = tid; idx < a.nbprev * 16; idx += 256) {
-      const int k = idx >> 4, r4 = (idx & 15) << 2;
+    // (a fixed trip count, so that all eight loads of a thread are in flight together)
+    float4 ev[B * 16 / 256];
+    const bool evec = (r0 + 63 < a.R) && ((a.R & 3) == 0);
+#pragma unroll
+    for (int it = 0; it < B * 16 / 256; ++it) {
+      const int idx = tid + it * 256;
+      const int k = min(idx >> 4, a.nbprev - 1), r4 = (idx & 15) << 2;
       const float* q = a.Eprev + (long)k * a.R;
-      float4 v;
-      if (r0 + r4 + 3 < a.R && ((a.R & 3) == 0)) {
-        v = *reinterpret_cast<const float4*>(q + r0 + r4);
+      if (evec) {
+        ev[it] = *reinterpret_cast<const float4*>(q + r0 + r4);
       } else {
-        v.x = q[min(r0 + r4 + 0, a.R - 1)];
-        v.y = q[min(r0 + r4 + 1, a.R - 1)];
-        v.z = q[min(r0 + r4 + 2, a.R - 1)];
-        v.w = q[min(r0 + r4 + 3, a.R - 1)];
+        ev[it].x = q[min(r0 + r4 + 0, a.R - 1)];
+        ev[it].y = q[min(r0 + r4 + 1, a.R - 1)];
+        ev[it].z = q[min(r0 + r4 + 2, a.R - 1)];
+        ev[it].w = q[min(r0 + r4 + 3, a.R - 1)];
       }
-      *reinterpret_cast<float4*>(&es[k * 64 + r4]) = v;
+    }
+#pragma unroll
+    for (int it = 0; it < B * 16 / 256; ++it) {
+      const int idx = tid + it * 256;
+      if ((idx >> 4) < a.nbprev) *reinterpret_cast<float4*>(&es[(idx >> 4) * 64 + ((idx & 15) << 2)]) = ev[it];
     }
     const int m = lane & 31, slot = lane >> 5;
     const int col = FULL ? (i1 + wave * 32 + m) : min(i1 + wave * 32 + m, a.C - 1);
@@ -178,8 +220,13 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   const int rd = a.rd;
   const int cend = FULL ? B : nb;
   cint_p srp = (cint_p)(a.scale_row);
+  // Micro-block m (columns 16m..16m+15) is walked by wavefront 0 while the other three fold the errors of
+  // micro-block m-1 into the columns beyond it; wavefront 0 folds those errors into its own 16 columns first and
+  // keeps them in registers for the walk.  The error buffer alternates, one barrier per micro-block.
 #pragma unroll 1
   for (int c0 = 0; c0 < cend; c0 += MB) {
+    const float* eprev = esh + (((c0 / MB) + 1) & 1) * MB * WSTRIDE;
+    float* ecur = esh + ((c0 / MB) & 1) * MB * WSTRIDE;
     if (wave == 0) {
       float w[MB], e[MB], sc[MB], zz[MB];
       float4 um[MB][MB / 4];
@@ -190,6 +237,12 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         sc[t] = a.scale[(long)srow * a.lds + r];
         zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
         w[t] = tile[(c0 + t) * WSTRIDE + lane];
+      }
+      if (c0 > 0) {
+        float ep[MB];
+#pragma unroll
+        for (int J = 0; J < MB; ++J) ep[J] = eprev[J * WSTRIDE + lane];
+        fold16(ut, ep, c0 - MB, c0, w);
       }
 #pragma unroll
       for (int J = 0; J < MB; ++J)
@@ -205,7 +258,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         q = fminf(fmaxf(q, 0.f), maxq);
         const float y = round_dtype((q - z) * s, rd);
         e[J] = (FULL || c0 + J < nb) ? (y - x) : 0.f;
-        esh[J * WSTRIDE + lane] = e[J];
+        ecur[J * WSTRIDE + lane] = e[J];
         if (FULL || c0 + J < nb) {
           wp[(long)(c0 + J) * a.ldw] = y;
           a.Qt[(long)(i1 + c0 + J) * a.R + r] = (uint8_t)q;
@@ -218,48 +271,17 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
           w[t] = fmaf(u, e[J], w[t]);
         }
       }
-    }
-    __syncthreads();
-    // fold the 16 errors into the remaining columns of the block, 16 columns per pass, passes dealt
-    // round-robin to the four wavefronts; U rows are fetched four at a time, one group ahead of the FMAs
-    if (c0 + MB + MB * wave < cend) {
+    } else if (c0 > 0 && c0 + MB * wave < cend) {
+      // passes of 16 columns beyond micro-block c0, dealt round-robin to wavefronts 1..3
       float e[MB];
 #pragma unroll
-      for (int J = 0; J < MB; ++J) e[J] = esh[J * WSTRIDE + lane];
+      for (int J = 0; J < MB; ++J) e[J] = eprev[J * WSTRIDE + lane];
 #pragma unroll 1
-      for (int k0 = c0 + MB + MB * wave; k0 < cend; k0 += 4 * MB) {
+      for (int k0 = c0 + MB * wave; k0 < cend; k0 += 3 * MB) {
         float x[MB];
-        float4 ug[2][4][MB / 4];
 #pragma unroll
         for (int t = 0; t < MB; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-          for (int t4 = 0; t4 < MB / 4; ++t4)
-            ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + jj, k0 + 4 * t4)]);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          if (g < 3) {
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-              for (int t4 = 0; t4 < MB / 4; ++t4)
-                ug[(g + 1) & 1][jj][t4] =
-                    *reinterpret_cast<const float4*>(&ut[ut_off(c0 + 4 * (g + 1) + jj, k0 + 4 * t4)]);
-          }
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            const float ej = e[4 * g + jj];
-#pragma unroll
-            for (int t4 = 0; t4 < MB / 4; ++t4) {
-              const float4 u = ug[g & 1][jj][t4];
-              x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
-              x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
-              x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
-              x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
-            }
-          }
-        }
+        fold16(ut, e, c0 - MB, k0, x);
 #pragma unroll
         for (int t = 0; t < MB; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
       }
@@ -268,7 +290,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   }
 }
 
-constexpr size_t COL_SMEM = (size_t)(B * WSTRIDE + UT_FLOATS + MB * WSTRIDE) * sizeof(float);
+constexpr size_t COL_SMEM = (size_t)(B * WSTRIDE + UT_FLOATS + 2 * MB * WSTRIDE) * sizeof(float);
 constexpr size_t BLOCK_SMEM = COL_SMEM > gemmf32::SMEM_BYTES ? COL_SMEM : gemmf32::SMEM_BYTES;
 
 template <bool ROWMAP, bool QZERO>
