@@ -96,12 +96,66 @@ __device__ __forceinline__ void fold16(const float* ut, const float (&e)[MB], in
   }
 }
 
+// The strictly sequential part: 16 columns of one row per lane, weights in w[].  Per column, the reference's
+// arithmetic: q = clamp(floor(x/s + z + 0.5), 0, maxq) with IEEE division, y = round_to(dtype)((q - z) * s),
+// e = y - x, then w[t] = fma(U[j,t], e, w[t]) for the columns t still to come.  RD: 0 fp32, 1 bf16, 2 fp16.
+// The multipliers U[j,t] (same for every lane) are fetched from LDS beforehand, all lanes on one address.
+// Each column's updates are issued at once and the scheduler is kept from moving work between columns: left
+// alone it postpones a column's updates until that column is walked, which puts up to 15 dependent multiply-adds
+// in front of every division.
+template <bool FULL, int RD>
+__device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], const float* ut,
+                                       int c0, int left, float maxq, float* esh_lane, float* wout, long ldw,
+                                       uint8_t* qout, float* eout, long R) {
+  float4 um[MB][MB / 4];
+#pragma unroll
+  for (int J = 0; J < MB; ++J)
+#pragma unroll
+    for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
+      um[J][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, c0 + 4 * t4)]);
+#pragma unroll
+  for (int J = 0; J < MB; ++J) {
+    const float s = sc[J], z = zz[J];
+    const float x = w[J];
+    const float v = x / s + z;
+    float q = floorf(v + 0.5f);
+    q = fminf(fmaxf(q, 0.f), maxq);
+    const float d = (q - z) * s;
+    float y = d;
+    if (RD == 1) {
+      // the hardware conversion rounds to nearest even like round_to_bf16; NaN stays NaN
+      y = (float)(__bf16)d;
+    } else if (RD == 2) {
+      y = __half2float(__float2half_rn(d));
+    }
+    const float e = (FULL || J < left) ? (y - x) : 0.f;
+    if (J + 1 < MB) {  // the next column first: it is the dependence chain
+      const float4 u4 = um[J][(J + 1) >> 2];
+      const float u = ((J + 1) & 3) == 0 ? u4.x : (((J + 1) & 3) == 1 ? u4.y : (((J + 1) & 3) == 2 ? u4.z : u4.w));
+      w[J + 1] = fmaf(u, e, w[J + 1]);
+    }
+    esh_lane[J * WSTRIDE] = e;
+    if (FULL || J < left) {
+      wout[(long)J * ldw] = y;
+      qout[(long)J * R] = (uint8_t)q;
+      eout[(long)J * R] = e;
+    }
+#pragma unroll
+    for (int t = J + 2; t < MB; ++t) {
+      const float4 u4 = um[J][t >> 2];
+      const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
+      w[t] = fmaf(u, e, w[t]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 // One workgroup (four wavefronts) owns 64 rows; lane l of every wavefront is row l.  The 128-column
 // block of those rows sits in LDS ([column][lane], so every access is conflict-free) next to the
 // 128x128 block of U.  16 columns at a time move to the registers of wavefront 0 for the strictly
-// sequential part; their 16 errors are published in LDS.  While wavefront 0 walks the next 16 columns (after
-// folding those errors into them itself), the other three wavefronts fold them into the rest of the block, each
-// taking every third pass of 16 columns.
+// sequential part; their 16 errors are published in LDS.  All four wavefronts fold them into the next 16 columns
+// at once; into the rest of the block the other three fold them while wavefront 0 walks those next 16 columns,
+// each taking every third pass of 16 columns.
 // For every weight the updates are applied in ascending j with one fma each, exactly the order of the
 // sequential reference.
 //
@@ -120,29 +174,35 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   float* tile = reinterpret_cast<float*>(smem);  // [B][WSTRIDE]
   float* ut = tile + B * WSTRIDE;                // packed upper micro-blocks of the U block
   float* esh = ut + UT_FLOATS;                   // [2][MB][WSTRIDE] errors of the current and the previous micro-block
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: row addresses below stay in scalar registers
   const int r0 = blockIdx.x * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
   // does, so no branch in this kernel ever diverges.
   const int r = min(r0 + lane, a.R - 1);
   float* __restrict__ wp = a.Wt + (long)i1 * a.ldw + r;
-  {
-    float t[32];  // each wavefront stages 32 of the 128 columns
+  // Every load of the set-up -- this block's weights, the previous block's errors, the two pieces of U -- is issued
+  // before the first of them is needed; nothing else runs on the CU to hide their latency.
+  float t[32];  // each wavefront stages 32 of the 128 columns
+  // (scalar row base + 32-bit lane offset: one address instruction per load instead of 64-bit vector arithmetic)
+  const unsigned ru = (unsigned)r;
 #pragma unroll
-    for (int k = 0; k < 32; ++k) t[k] = (FULL || wave * 32 + k < nb) ? wp[(long)(wave * 32 + k) * a.ldw] : 0.f;
-#pragma unroll
-    for (int k = 0; k < 32; ++k) tile[(wave * 32 + k) * WSTRIDE + lane] = t[k];
+  for (int k = 0; k < 32; ++k) {
+    const float* rowp = a.Wt + (long)(i1 + min(wave * 32 + k, nb - 1)) * a.ldw;
+    const float v = rowp[ru];
+    t[k] = (FULL || wave * 32 + k < nb) ? v : 0.f;
   }
-  if (a.Eprev) {
-    // The previous block's errors, folded into this block's columns:
-    //   tile[c][row] += sum_k U[i1-nbprev+k, i1+c] * Eprev[k][row].
-    // Wavefront w takes columns 32w..32w+31 and all 64 rows: two 32x32 accumulators.  The errors (shared by the
-    // four wavefronts) are staged in the LDS area the U block will occupy afterwards; the U operand comes
-    // straight from memory in MFMA layout (lane = column, the two k of an instruction in the two lane halves),
-    // every load issued before the first product.
-    float* es = ut;  // [nbprev][64]
-    // (a fixed trip count, so that all eight loads of a thread are in flight together)
-    float4 ev[B * 16 / 256];
+  const bool pre = a.Eprev != nullptr;
+  // The previous block's errors, folded into this block's columns:
+  //   tile[c][row] += sum_k U[i1-nbprev+k, i1+c] * Eprev[k][row].
+  // Wavefront w takes columns 32w..32w+31 and all 64 rows: two 32x32 accumulators.  The errors (shared by the
+  // four wavefronts) are staged in the LDS area the U block will occupy afterwards; the U operand comes
+  // straight from memory in MFMA layout (lane = column, the two k of an instruction in the two lane halves).
+  float* es = ut;  // [nbprev][64]
+  const int m = lane & 31, slot = lane >> 5;
+  float4 ev[B * 16 / 256];
+  float av[B / 2];
+  if (pre) {
     const bool evec = (r0 + 63 < a.R) && ((a.R & 3) == 0);
 #pragma unroll
     for (int it = 0; it < B * 16 / 256; ++it) {
@@ -158,30 +218,52 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         ev[it].w = q[min(r0 + r4 + 3, a.R - 1)];
       }
     }
+    const int col = FULL ? (wave * 32 + m) : min(wave * 32 + m, a.C - 1 - i1);
+    if (a.nbprev == B) {  // the usual case: scalar row base, the lane adds its column and its k slot
+      const unsigned off = (unsigned)(slot * (int)a.ldu + col);
+#pragma unroll
+      for (int tt = 0; tt < B / 2; ++tt) {
+        const float* rowp = a.U + (long)(i1 - B + 2 * tt) * a.ldu + i1;
+        av[tt] = rowp[off];
+      }
+    } else {
+      const float* __restrict__ Uo = a.U + (long)(i1 - a.nbprev) * a.ldu + i1 + col;
+#pragma unroll
+      for (int tt = 0; tt < B / 2; ++tt) {
+        const int k = 2 * tt + slot;
+        const float v = Uo[(long)min(k, a.nbprev - 1) * a.ldu];
+        av[tt] = k < a.nbprev ? v : 0.f;
+      }
+    }
+  }
+  const float* __restrict__ Ub = a.U + (long)i1 * a.ldu + i1;
+  const bool vec = FULL && ((a.ldu & 3) == 0) && ((((uintptr_t)Ub) & 15) == 0);
+  float4 uv[16];
+  if (vec) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int idx = tid + u * 256;
+      const int j = idx >> 5, k = (idx & 31) << 2;
+      uv[u] = (k + 3 > j) ? *reinterpret_cast<const float4*>(Ub + (long)j * a.ldu + k) : make_float4(0, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 32; ++k) tile[(wave * 32 + k) * WSTRIDE + lane] = t[k];
+  if (pre) {
 #pragma unroll
     for (int it = 0; it < B * 16 / 256; ++it) {
       const int idx = tid + it * 256;
       if ((idx >> 4) < a.nbprev) *reinterpret_cast<float4*>(&es[(idx >> 4) * 64 + ((idx & 15) << 2)]) = ev[it];
-    }
-    const int m = lane & 31, slot = lane >> 5;
-    const int col = FULL ? (i1 + wave * 32 + m) : min(i1 + wave * 32 + m, a.C - 1);
-    const float* __restrict__ Uo = a.U + (long)(i1 - a.nbprev) * a.ldu + col;
-    float av[B / 2];
-#pragma unroll
-    for (int t = 0; t < B / 2; ++t) {
-      const int k = 2 * t + slot;
-      const float v = Uo[(long)min(k, a.nbprev - 1) * a.ldu];
-      av[t] = k < a.nbprev ? v : 0.f;
     }
     floatx16 acc0, acc1;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
     __syncthreads();
 #pragma unroll
-    for (int t = 0; t < B / 2; ++t) {
-      const int k = min(2 * t + slot, a.nbprev - 1);  // rows past nbprev meet a zero multiplier
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], es[k * 64 + m], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], es[k * 64 + 32 + m], acc1, 0, 0, 0);
+    for (int tt = 0; tt < B / 2; ++tt) {
+      const int k = min(2 * tt + slot, a.nbprev - 1);  // rows past nbprev meet a zero multiplier
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[tt], es[k * 64 + m], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(av[tt], es[k * 64 + 32 + m], acc1, 0, 0, 0);
     }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -191,28 +273,17 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
     }
     __syncthreads();  // es is about to be overwritten by the U block
   }
-  {
-    const float* __restrict__ Ub = a.U + (long)i1 * a.ldu + i1;
-    const bool vec = FULL && ((a.ldu & 3) == 0) && ((((uintptr_t)Ub) & 15) == 0);
-    if (vec) {
-      float4 v[16];
+  if (vec) {
 #pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int idx = tid + u * 256;
-        const int j = idx >> 5, k = (idx & 31) << 2;
-        v[u] = (k + 3 > j) ? *reinterpret_cast<const float4*>(Ub + (long)j * a.ldu + k) : make_float4(0, 0, 0, 0);
-      }
-#pragma unroll
-      for (int u = 0; u < 16; ++u) {
-        const int idx = tid + u * 256;
-        const int j = idx >> 5, k = (idx & 31) << 2;
-        if ((k >> 4) >= (j >> 4)) *reinterpret_cast<float4*>(&ut[ut_off(j, k)]) = v[u];
-      }
-    } else {
-      for (int idx = tid; idx < B * B; idx += 256) {
-        const int j = idx >> 7, k = idx & 127;
-        if ((k >> 4) >= (j >> 4)) ut[ut_off(j, k)] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
-      }
+    for (int u = 0; u < 16; ++u) {
+      const int idx = tid + u * 256;
+      const int j = idx >> 5, k = (idx & 31) << 2;
+      if ((k >> 4) >= (j >> 4)) *reinterpret_cast<float4*>(&ut[ut_off(j, k)]) = uv[u];
+    }
+  } else {
+    for (int idx = tid; idx < B * B; idx += 256) {
+      const int j = idx >> 7, k = idx & 127;
+      if ((k >> 4) >= (j >> 4)) ut[ut_off(j, k)] = (j < nb && k < nb && k > j) ? Ub[(long)j * a.ldu + k] : 0.f;
     }
   }
   __syncthreads();
@@ -221,15 +292,14 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   const int cend = FULL ? B : nb;
   cint_p srp = (cint_p)(a.scale_row);
   // Micro-block m (columns 16m..16m+15) is walked by wavefront 0 while the other three fold the errors of
-  // micro-block m-1 into the columns beyond it; wavefront 0 folds those errors into its own 16 columns first and
-  // keeps them in registers for the walk.  The error buffer alternates, one barrier per micro-block.
+  // micro-block m-1 into the columns beyond m.  Then all four fold the errors of m into the 16 columns of m+1 (the
+  // only fold the next walk has to wait for, a quarter each).  The error buffer alternates.
 #pragma unroll 1
   for (int c0 = 0; c0 < cend; c0 += MB) {
     const float* eprev = esh + (((c0 / MB) + 1) & 1) * MB * WSTRIDE;
     float* ecur = esh + ((c0 / MB) & 1) * MB * WSTRIDE;
     if (wave == 0) {
-      float w[MB], e[MB], sc[MB], zz[MB];
-      float4 um[MB][MB / 4];
+      float w[MB], sc[MB], zz[MB];
 #pragma unroll
       for (int t = 0; t < MB; ++t) {
         const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
@@ -238,41 +308,17 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
         w[t] = tile[(c0 + t) * WSTRIDE + lane];
       }
-      if (c0 > 0) {
-        float ep[MB];
-#pragma unroll
-        for (int J = 0; J < MB; ++J) ep[J] = eprev[J * WSTRIDE + lane];
-        fold16(ut, ep, c0 - MB, c0, w);
-      }
-#pragma unroll
-      for (int J = 0; J < MB; ++J)
-#pragma unroll
-        for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
-          um[J][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, c0 + 4 * t4)]);
-#pragma unroll
-      for (int J = 0; J < MB; ++J) {
-        const float s = sc[J], z = zz[J];
-        const float x = w[J];
-        const float v = x / s + z;
-        float q = floorf(v + 0.5f);
-        q = fminf(fmaxf(q, 0.f), maxq);
-        const float y = round_dtype((q - z) * s, rd);
-        e[J] = (FULL || c0 + J < nb) ? (y - x) : 0.f;
-        ecur[J * WSTRIDE + lane] = e[J];
-        if (FULL || c0 + J < nb) {
-          wp[(long)(c0 + J) * a.ldw] = y;
-          a.Qt[(long)(i1 + c0 + J) * a.R + r] = (uint8_t)q;
-          a.E[(long)(c0 + J) * a.R + r] = e[J];
-        }
-#pragma unroll
-        for (int t = J + 1; t < MB; ++t) {
-          const float4 u4 = um[J][t >> 2];
-          const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
-          w[t] = fmaf(u, e[J], w[t]);
-        }
-      }
+      const float* utd = ut;
+      float* wout = wp + (long)c0 * a.ldw;
+      uint8_t* qout = a.Qt + (long)(i1 + c0) * a.R + r;
+      float* eout = a.E + (long)c0 * a.R + r;
+      const int left = nb - c0;  // columns of the block from c0 on
+      if (rd == 1) walk16<FULL, 1>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
+      else if (rd == 2) walk16<FULL, 2>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
+      else walk16<FULL, 0>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
     } else if (c0 > 0 && c0 + MB * wave < cend) {
-      // passes of 16 columns beyond micro-block c0, dealt round-robin to wavefronts 1..3
+      // the previous micro-block's errors: passes of 16 columns beyond micro-block c0, dealt round-robin to
+      // wavefronts 1..3
       float e[MB];
 #pragma unroll
       for (int J = 0; J < MB; ++J) e[J] = eprev[J * WSTRIDE + lane];
@@ -285,6 +331,31 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
 #pragma unroll
         for (int t = 0; t < MB; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
       }
+    }
+    __syncthreads();
+    // this micro-block's errors into the next micro-block's columns, the only ones the walk needs at once: four
+    // columns per wavefront (they already hold the previous micro-block's contribution, ascending j as ever)
+    if (c0 + MB < cend) {
+      const int k0 = c0 + MB + 4 * wave;
+      float x[4];
+      float4 u[MB];
+      float ej[MB];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
+#pragma unroll
+      for (int J = 0; J < MB; ++J) {
+        u[J] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, k0)]);
+        ej[J] = ecur[J * WSTRIDE + lane];
+      }
+#pragma unroll
+      for (int J = 0; J < MB; ++J) {
+        x[0] = fmaf(u[J].x, ej[J], x[0]);
+        x[1] = fmaf(u[J].y, ej[J], x[1]);
+        x[2] = fmaf(u[J].z, ej[J], x[2]);
+        x[3] = fmaf(u[J].w, ej[J], x[3]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
     }
     __syncthreads();
   }
