@@ -294,20 +294,42 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   // Micro-block m (columns 16m..16m+15) is walked by wavefront 0 while the other three fold the errors of
   // micro-block m-1 into the columns beyond m.  Then all four fold the errors of m into the 16 columns of m+1 (the
   // only fold the next walk has to wait for, a quarter each).  The error buffer alternates.
+  // With one scale row for the whole block (grouped scales, a group at least as wide as the block) the scale and
+  // zero point are read once instead of per micro-block.
+  bool one_row = false;
+  float sc_blk = 0.f, zz_blk = 0.f;
+  if (ROWMAP) {
+    const int s0 = srp[i1];
+    const int sa = a.scale_row[i1 + min(lane, cend - 1)], sb = a.scale_row[i1 + min(64 + lane, cend - 1)];
+    one_row = __ballot(sa != s0 || sb != s0) == 0;  // every wavefront looks at all 128 entries: same answer in each
+    if (one_row) {
+      sc_blk = a.scale[(long)s0 * a.lds + r];
+      zz_blk = QZERO ? a.qzero[(long)s0 * a.lds + r] : a.qzero_const;
+    }
+  }
 #pragma unroll 1
   for (int c0 = 0; c0 < cend; c0 += MB) {
     const float* eprev = esh + (((c0 / MB) + 1) & 1) * MB * WSTRIDE;
     float* ecur = esh + ((c0 / MB) & 1) * MB * WSTRIDE;
     if (wave == 0) {
       float w[MB], sc[MB], zz[MB];
+      if (one_row) {
 #pragma unroll
-      for (int t = 0; t < MB; ++t) {
-        const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
-        const int srow = ROWMAP ? srp[col] : col;
-        sc[t] = a.scale[(long)srow * a.lds + r];
-        zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
-        w[t] = tile[(c0 + t) * WSTRIDE + lane];
+        for (int t = 0; t < MB; ++t) {
+          sc[t] = sc_blk;
+          zz[t] = zz_blk;
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < MB; ++t) {
+          const int col = FULL ? (i1 + c0 + t) : min(i1 + c0 + t, a.C - 1);
+          const int srow = ROWMAP ? srp[col] : col;
+          sc[t] = a.scale[(long)srow * a.lds + r];
+          zz[t] = QZERO ? a.qzero[(long)srow * a.lds + r] : a.qzero_const;
+        }
       }
+#pragma unroll
+      for (int t = 0; t < MB; ++t) w[t] = tile[(c0 + t) * WSTRIDE + lane];
       const float* utd = ut;
       float* wout = wp + (long)c0 * a.ldw;
       uint8_t* qout = a.Qt + (long)(i1 + c0) * a.R + r;
