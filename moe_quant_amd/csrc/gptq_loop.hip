@@ -103,21 +103,36 @@ __device__ __forceinline__ void fold16(const float* ut, const float (&e)[MB], in
 // Each column's updates are issued at once and the scheduler is kept from moving work between columns: left
 // alone it postpones a column's updates until that column is walked, which puts up to 15 dependent multiply-adds
 // in front of every division.
-template <bool FULL, int RD>
-__device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], const float* ut,
-                                       int c0, int left, float maxq, float* esh_lane, float* wout, long ldw,
-                                       uint8_t* qout, float* eout, long R) {
+template <bool FULL, int RD, bool RCP>
+__device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], float rcp_blk,
+                                       const float* ut, int c0, int left, float maxq, float* esh_lane, float* wout,
+                                       long ldw, uint8_t* qout, float* eout, long R) {
   float4 um[MB][MB / 4];
 #pragma unroll
   for (int J = 0; J < MB; ++J)
 #pragma unroll
     for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
       um[J][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, c0 + 4 * t4)]);
+  // x / s with IEEE rounding, three dependent operations instead of the division's eleven: with rcp = RN(1/s)
+  // (a true division, but off the chain: s is known beforehand), q0 = RN(x*rcp), the exact remainder x - q0*s
+  // (one fma) and q1 = RN(q0 + rem*rcp) is the correctly rounded quotient (Markstein).  Where that argument does
+  // not apply -- s = 0 or so small that rcp overflows, a quotient beyond the fp32 range -- q0 already is what the
+  // division gives (an infinity or NaN), and is kept.
+  // Used when one reciprocal serves the whole block (RCP: rcp_blk = 1/s computed once by the caller); with a scale
+  // per column the 16 reciprocals would cost more than they save.
 #pragma unroll
   for (int J = 0; J < MB; ++J) {
     const float s = sc[J], z = zz[J];
     const float x = w[J];
-    const float v = x / s + z;
+    float quot;
+    if (RCP) {
+      const float q0 = x * rcp_blk;
+      const float q1 = fmaf(fmaf(-q0, s, x), rcp_blk, q0);
+      quot = fabsf(q0) < 3.0e38f ? q1 : q0;
+    } else {
+      quot = x / s;
+    }
+    const float v = quot + z;
     float q = floorf(v + 0.5f);
     q = fminf(fmaxf(q, 0.f), maxq);
     const float d = (q - z) * s;
@@ -297,7 +312,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
   // With one scale row for the whole block (grouped scales, a group at least as wide as the block) the scale and
   // zero point are read once instead of per micro-block.
   bool one_row = false;
-  float sc_blk = 0.f, zz_blk = 0.f;
+  float sc_blk = 0.f, zz_blk = 0.f, rcp_blk = 0.f;
   if (ROWMAP) {
     const int s0 = srp[i1];
     const int sa = a.scale_row[i1 + min(lane, cend - 1)], sb = a.scale_row[i1 + min(64 + lane, cend - 1)];
@@ -305,6 +320,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
     if (one_row) {
       sc_blk = a.scale[(long)s0 * a.lds + r];
       zz_blk = QZERO ? a.qzero[(long)s0 * a.lds + r] : a.qzero_const;
+      rcp_blk = 1.0f / sc_blk;
     }
   }
 #pragma unroll 1
@@ -335,9 +351,18 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
       uint8_t* qout = a.Qt + (long)(i1 + c0) * a.R + r;
       float* eout = a.E + (long)c0 * a.R + r;
       const int left = nb - c0;  // columns of the block from c0 on
-      if (rd == 1) walk16<FULL, 1>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
-      else if (rd == 2) walk16<FULL, 2>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
-      else walk16<FULL, 0>(w, sc, zz, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R);
+#define MQ_WALK(RD_, RCP_) \
+  walk16<FULL, RD_, RCP_>(w, sc, zz, rcp_blk, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R)
+      if (one_row) {
+        if (rd == 1) MQ_WALK(1, true);
+        else if (rd == 2) MQ_WALK(2, true);
+        else MQ_WALK(0, true);
+      } else {
+        if (rd == 1) MQ_WALK(1, false);
+        else if (rd == 2) MQ_WALK(2, false);
+        else MQ_WALK(0, false);
+      }
+#undef MQ_WALK
     } else if (c0 > 0 && c0 + MB * wave < cend) {
       // the previous micro-block's errors: passes of 16 columns beyond micro-block c0, dealt round-robin to
       // wavefronts 1..3
