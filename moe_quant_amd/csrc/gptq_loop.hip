@@ -62,107 +62,123 @@ constexpr int UT_FLOATS = 36 * 256;
 
 typedef const int __attribute__((address_space(4))) * cint_p;  // constant address space: scalar loads
 
-// x[t] += sum_J U[j0+J, k0+t] * e[J] for the 16 columns k0.. and the 16 errors of columns j0.. (ascending J, one fma
-// each).  The multipliers are the same for every lane: read from LDS with all lanes on one address (a broadcast,
-// four values per read), four rows of U at a time, one group ahead of the FMAs.  (Scalar loads of U from memory,
-// which would keep the multipliers out of the vector registers, measured slower: they wait on L2.)
-__device__ __forceinline__ void fold16(const float* ut, const float (&e)[MB], int j0, int k0, float (&x)[MB]) {
-  float4 ug[2][4][MB / 4];
-#pragma unroll
-  for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-    for (int t4 = 0; t4 < MB / 4; ++t4) ug[0][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(j0 + jj, k0 + 4 * t4)]);
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    if (g < 3) {
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int t4 = 0; t4 < MB / 4; ++t4)
-          ug[(g + 1) & 1][jj][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(j0 + 4 * (g + 1) + jj, k0 + 4 * t4)]);
-    }
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const float ej = e[4 * g + jj];
-#pragma unroll
-      for (int t4 = 0; t4 < MB / 4; ++t4) {
-        const float4 u = ug[g & 1][jj][t4];
-        x[4 * t4 + 0] = fmaf(u.x, ej, x[4 * t4 + 0]);
-        x[4 * t4 + 1] = fmaf(u.y, ej, x[4 * t4 + 1]);
-        x[4 * t4 + 2] = fmaf(u.z, ej, x[4 * t4 + 2]);
-        x[4 * t4 + 3] = fmaf(u.w, ej, x[4 * t4 + 3]);
-      }
+// acc += rep[lane N of this lane's row of 16 lanes] * v in one instruction: the multiplier comes through a DPP row
+// broadcast.  FIRST: the two wait states required between the instruction that wrote rep and a DPP read of it (the
+// compiler cannot see that this statement is a DPP instruction).
+template <int N, bool FIRST>
+__device__ __forceinline__ void fmac_rowbcast(float& acc, float rep, float v) {
+  if (FIRST)
+    asm("s_nop 1\n\tv_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(rep), "v"(v), "n"(N));
+  else
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(rep), "v"(v), "n"(N));
+}
+template <int T, int N>
+struct RowFma {  // x[T..N-1] += u[lane T.. of the row] * e
+  static __device__ __forceinline__ void run(float (&x)[MB], float u, float e) {
+    if constexpr (T < N) {
+      fmac_rowbcast<T, T == 0>(x[T], u, e);
+      RowFma<T + 1, N>::run(x, u, e);
     }
   }
+};
+
+// x[t] += sum_J U[j0+J, k0+t] * e[J] for the 16 columns k0.. and the 16 errors of columns j0.. (ascending J, one
+// fused multiply-add each).  The multipliers are the same for every lane.  Row J of the 16x16 block of U is read
+// from LDS once, lane l taking element l%16 (so each row of 16 lanes holds the whole row of U), and every product
+// takes its multiplier from there through a DPP row broadcast: 16 LDS reads per pass instead of 64, and nothing
+// but the multiply-adds in between.  (Scalar loads of U from memory measured slower: they wait on L2.)
+__device__ __forceinline__ void fold16(const float* ut, const float (&e)[MB], int j0, int k0, float (&x)[MB], int lane) {
+  float u[MB];
+#pragma unroll
+  for (int J = 0; J < MB; ++J) u[J] = ut[ut_off(j0 + J, k0) + (lane & 15)];
+#pragma unroll
+  for (int J = 0; J < MB; ++J) RowFma<0, MB>::run(x, u[J], e[J]);
 }
 
 // The strictly sequential part: 16 columns of one row per lane, weights in w[].  Per column, the reference's
 // arithmetic: q = clamp(floor(x/s + z + 0.5), 0, maxq) with IEEE division, y = round_to(dtype)((q - z) * s),
 // e = y - x, then w[t] = fma(U[j,t], e, w[t]) for the columns t still to come.  RD: 0 fp32, 1 bf16, 2 fp16.
-// The multipliers U[j,t] (same for every lane) are fetched from LDS beforehand, all lanes on one address.
+// The multipliers U[j,t] (same for every lane) come from u[j], which holds row j of the 16x16 block of U in every row
+// of 16 lanes, through DPP row broadcasts: one instruction per update.
 // Each column's updates are issued at once and the scheduler is kept from moving work between columns: left
 // alone it postpones a column's updates until that column is walked, which puts up to 15 dependent multiply-adds
 // in front of every division.
-template <bool FULL, int RD, bool RCP>
-__device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], float rcp_blk,
-                                       const float* ut, int c0, int left, float maxq, float* esh_lane, float* wout,
-                                       long ldw, uint8_t* qout, float* eout, long R) {
-  float4 um[MB][MB / 4];
-#pragma unroll
-  for (int J = 0; J < MB; ++J)
-#pragma unroll
-    for (int t4 = (J + 1) / 4; t4 < MB / 4; ++t4)
-      um[J][t4] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, c0 + 4 * t4)]);
-  // x / s with IEEE rounding, three dependent operations instead of the division's eleven: with rcp = RN(1/s)
-  // (a true division, but off the chain: s is known beforehand), q0 = RN(x*rcp), the exact remainder x - q0*s
-  // (one fma) and q1 = RN(q0 + rem*rcp) is the correctly rounded quotient (Markstein).  Where that argument does
-  // not apply -- s = 0 or so small that rcp overflows, a quotient beyond the fp32 range -- q0 already is what the
-  // division gives (an infinity or NaN), and is kept.
-  // Used when one reciprocal serves the whole block (RCP: rcp_blk = 1/s computed once by the caller); with a scale
-  // per column the 16 reciprocals would cost more than they save.
-#pragma unroll
-  for (int J = 0; J < MB; ++J) {
-    const float s = sc[J], z = zz[J];
-    const float x = w[J];
-    float quot;
-    if (RCP) {
-      const float q0 = x * rcp_blk;
-      const float q1 = fmaf(fmaf(-q0, s, x), rcp_blk, q0);
-      quot = fabsf(q0) < 3.0e38f ? q1 : q0;
-    } else {
-      quot = x / s;
+//
+// x / s with IEEE rounding, three dependent operations instead of the division's eleven (RCP): with rcp = RN(1/s)
+// (a true division, but off the chain: s is known beforehand), q0 = RN(x*rcp), the exact remainder x - q0*s
+// (one fma) and q1 = RN(q0 + rem*rcp) is the correctly rounded quotient (Markstein).  Where that argument does
+// not apply -- s = 0 or so small that rcp overflows, a quotient beyond the fp32 range -- q0 already is what the
+// division gives (an infinity or NaN), and is kept.  Used when one reciprocal serves the whole block (rcp_blk =
+// 1/s computed once by the caller); with a scale per column the 16 reciprocals would cost more than they save.
+struct WalkCtx {
+  float rcp_blk, maxq;
+  int left;  // columns of the block from this micro-block's first on
+  float* esh_lane;
+  float* wout;
+  long ldw;
+  uint8_t* qout;
+  float* eout;
+  long R;
+};
+
+template <int T, int J>
+struct WalkFma {  // w[T..15] += U[j, T..] * e
+  static __device__ __forceinline__ void run(float (&w)[MB], float u, float e) {
+    if constexpr (T < MB) {
+      fmac_rowbcast<T, T == J + 1>(w[T], u, e);
+      WalkFma<T + 1, J>::run(w, u, e);
     }
-    const float v = quot + z;
-    float q = floorf(v + 0.5f);
-    q = fminf(fmaxf(q, 0.f), maxq);
-    const float d = (q - z) * s;
-    float y = d;
-    if (RD == 1) {
-      // the hardware conversion rounds to nearest even like round_to_bf16; NaN stays NaN
-      y = (float)(__bf16)d;
-    } else if (RD == 2) {
-      y = __half2float(__float2half_rn(d));
-    }
-    const float e = (FULL || J < left) ? (y - x) : 0.f;
-    if (J + 1 < MB) {  // the next column first: it is the dependence chain
-      const float4 u4 = um[J][(J + 1) >> 2];
-      const float u = ((J + 1) & 3) == 0 ? u4.x : (((J + 1) & 3) == 1 ? u4.y : (((J + 1) & 3) == 2 ? u4.z : u4.w));
-      w[J + 1] = fmaf(u, e, w[J + 1]);
-    }
-    esh_lane[J * WSTRIDE] = e;
-    if (FULL || J < left) {
-      wout[(long)J * ldw] = y;
-      qout[(long)J * R] = (uint8_t)q;
-      eout[(long)J * R] = e;
-    }
-#pragma unroll
-    for (int t = J + 2; t < MB; ++t) {
-      const float4 u4 = um[J][t >> 2];
-      const float u = (t & 3) == 0 ? u4.x : ((t & 3) == 1 ? u4.y : ((t & 3) == 2 ? u4.z : u4.w));
-      w[t] = fmaf(u, e, w[t]);
-    }
-    __builtin_amdgcn_sched_barrier(0);
   }
+};
+
+template <bool FULL, int RD, bool RCP, int J>
+struct WalkStep {
+  static __device__ __forceinline__ void run(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB],
+                                             const float (&u)[MB], const WalkCtx& c) {
+    if constexpr (J < MB) {
+      const float s = sc[J], z = zz[J];
+      const float x = w[J];
+      float quot;
+      if (RCP) {
+        const float q0 = x * c.rcp_blk;
+        const float q1 = fmaf(fmaf(-q0, s, x), c.rcp_blk, q0);
+        quot = fabsf(q0) < 3.0e38f ? q1 : q0;
+      } else {
+        quot = x / s;
+      }
+      const float v = quot + z;
+      float q = floorf(v + 0.5f);
+      q = fminf(fmaxf(q, 0.f), c.maxq);
+      const float d = (q - z) * s;
+      float y = d;
+      if (RD == 1) {
+        y = (float)(__bf16)d;  // the hardware conversion rounds to nearest even like round_to_bf16; NaN stays NaN
+      } else if (RD == 2) {
+        y = __half2float(__float2half_rn(d));
+      }
+      const float e = (FULL || J < c.left) ? (y - x) : 0.f;
+      WalkFma<J + 1, J>::run(w, u[J], e);  // the next column first: it is the dependence chain
+      c.esh_lane[J * WSTRIDE] = e;
+      if (FULL || J < c.left) {
+        c.wout[(long)J * c.ldw] = y;
+        c.qout[(long)J * c.R] = (uint8_t)q;
+        c.eout[(long)J * c.R] = e;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      WalkStep<FULL, RD, RCP, J + 1>::run(w, sc, zz, u, c);
+    }
+  }
+};
+
+template <bool FULL, int RD, bool RCP>
+__device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], const float* ut,
+                                       int c0, int lane, const WalkCtx& c) {
+  float u[MB];  // row J of the micro-block of U: lane l holds U[c0+J, c0 + l%16]
+#pragma unroll
+  for (int J = 0; J < MB; ++J) u[J] = ut[ut_off(c0 + J, c0) + (lane & 15)];
+  WalkStep<FULL, RD, RCP, 0>::run(w, sc, zz, u, c);
 }
 
 // One workgroup (four wavefronts) owns 64 rows; lane l of every wavefront is row l.  The 128-column
@@ -347,12 +363,9 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
 #pragma unroll
       for (int t = 0; t < MB; ++t) w[t] = tile[(c0 + t) * WSTRIDE + lane];
       const float* utd = ut;
-      float* wout = wp + (long)c0 * a.ldw;
-      uint8_t* qout = a.Qt + (long)(i1 + c0) * a.R + r;
-      float* eout = a.E + (long)c0 * a.R + r;
-      const int left = nb - c0;  // columns of the block from c0 on
-#define MQ_WALK(RD_, RCP_) \
-  walk16<FULL, RD_, RCP_>(w, sc, zz, rcp_blk, utd, c0, left, maxq, ecur + lane, wout, a.ldw, qout, eout, a.R)
+      const WalkCtx wc{rcp_blk, maxq, nb - c0, ecur + lane, wp + (long)c0 * a.ldw, a.ldw,
+                       a.Qt + (long)(i1 + c0) * a.R + r, a.E + (long)c0 * a.R + r, a.R};
+#define MQ_WALK(RD_, RCP_) walk16<FULL, RD_, RCP_>(w, sc, zz, utd, c0, lane, wc)
       if (one_row) {
         if (rd == 1) MQ_WALK(1, true);
         else if (rd == 2) MQ_WALK(2, true);
@@ -374,7 +387,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
         float x[MB];
 #pragma unroll
         for (int t = 0; t < MB; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
-        fold16(ut, e, c0 - MB, k0, x);
+        fold16(ut, e, c0 - MB, k0, x, lane);
 #pragma unroll
         for (int t = 0; t < MB; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
       }
@@ -385,21 +398,22 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int
     if (c0 + MB < cend) {
       const int k0 = c0 + MB + 4 * wave;
       float x[4];
-      float4 u[MB];
+      float u[MB];  // row J of the block of U above the next micro-block, rotated so that lane 0..3 of a row of 16 hold
+                    // this wavefront's four columns
       float ej[MB];
 #pragma unroll
       for (int t = 0; t < 4; ++t) x[t] = tile[(k0 + t) * WSTRIDE + lane];
 #pragma unroll
       for (int J = 0; J < MB; ++J) {
-        u[J] = *reinterpret_cast<const float4*>(&ut[ut_off(c0 + J, k0)]);
+        u[J] = ut[ut_off(c0 + J, c0 + MB) + ((lane + 4 * wave) & 15)];
         ej[J] = ecur[J * WSTRIDE + lane];
       }
 #pragma unroll
       for (int J = 0; J < MB; ++J) {
-        x[0] = fmaf(u[J].x, ej[J], x[0]);
-        x[1] = fmaf(u[J].y, ej[J], x[1]);
-        x[2] = fmaf(u[J].z, ej[J], x[2]);
-        x[3] = fmaf(u[J].w, ej[J], x[3]);
+        fmac_rowbcast<0, true>(x[0], u[J], ej[J]);
+        fmac_rowbcast<1, false>(x[1], u[J], ej[J]);
+        fmac_rowbcast<2, false>(x[2], u[J], ej[J]);
+        fmac_rowbcast<3, false>(x[3], u[J], ej[J]);
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t) tile[(k0 + t) * WSTRIDE + lane] = x[t];
