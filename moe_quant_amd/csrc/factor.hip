@@ -336,6 +336,79 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void r
   diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false);
 }
 
+// The next diagonal tile, brought up to date by one workgroup on its own:  S(r,c) = H(r,c) - sum_k P(r,k) P(c,k)
+// for the 128x128 tile at (i1-128, i1-128), P = A[i1-128 : i1, i1 : i1+128] (the panel rows of that block).
+// It sits on the dependence chain of every step, so it is not run as a generic GEMM tile: all of P goes to LDS
+// once (64 KB, one barrier instead of one per K slice), only the ten 32x32 sub-tiles on or above the diagonal are
+// formed, dealt 3/3/2/2 to the four wavefronts (12k instead of 16k matrix-core cycles), operands and results
+// move 16 bytes at a time (transposed accumulators, as in tile_update), and the old tile is added row-wise from
+// registers loaded at the very start.  The result lands in the S position of buf; left of a row's diagonal is junk.
+__device__ __forceinline__ void diag_tile_update(float* buf, const float* A, long ld, int i1) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const float* P = A + (long)(i1 - NB) * ld + i1;
+  const float* H = A + (long)(i1 - NB) * ld + (i1 - NB);
+  floatx4 pv[16], hv[16];
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256;
+    pv[it] = *reinterpret_cast<const floatx4*>(P + (long)(idx >> 5) * ld + ((idx & 31) << 2));
+  }
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256;
+    hv[it] = *reinterpret_cast<const floatx4*>(H + (long)(idx >> 5) * ld + ((idx & 31) << 2));
+  }
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256;
+    *reinterpret_cast<floatx4*>(buf + (idx >> 5) * LDM + ((idx & 31) << 2)) = pv[it];
+  }
+  __syncthreads();
+  const int x = lane & 31, h = lane >> 5;
+  // sub-tile list (row block, column block): wavefront w takes entries w, w+4, w+8
+  constexpr int TI = 0x21110000, TJ = 0x23213210;  // nibble n: entry n (entries 0..7); entries 8, 9 below
+  floatx16 acc[3];
+#pragma unroll
+  for (int s3 = 0; s3 < 3; ++s3) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[s3][v] = 0.f;
+    const int e = wave + 4 * s3;
+    if (e < 10) {
+      const int I = e < 8 ? ((TI >> (4 * e)) & 15) : (e == 8 ? 2 : 3), Jc = e < 8 ? ((TJ >> (4 * e)) & 15) : 3;
+      const float* pa = buf + (SB * I + x) * LDM + 4 * h;
+      const float* pb = buf + (SB * Jc + x) * LDM + 4 * h;
+#pragma unroll
+      for (int j = 0; j < NB / 8; ++j) {
+        const floatx4 a4 = *reinterpret_cast<const floatx4*>(pa + 8 * j);
+        const floatx4 b4 = *reinterpret_cast<const floatx4*>(pb + 8 * j);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[s3] = __builtin_amdgcn_mfma_f32_32x32x2f32(b4[t], a4[t], acc[s3], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();  // every wavefront is done reading P: its place is taken by the result
+#pragma unroll
+  for (int s3 = 0; s3 < 3; ++s3) {
+    const int e = wave + 4 * s3;
+    if (e < 10) {
+      const int I = e < 8 ? ((TI >> (4 * e)) & 15) : (e == 8 ? 2 : 3), Jc = e < 8 ? ((TJ >> (4 * e)) & 15) : 3;
+      float* pc = buf + (SB * I + x) * LDM + SOFF + SB * Jc + 4 * h;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const floatx4 t = {-acc[s3][4 * g], -acc[s3][4 * g + 1], -acc[s3][4 * g + 2], -acc[s3][4 * g + 3]};
+        *reinterpret_cast<floatx4*>(pc + 8 * g) = t;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256;
+    floatx4* q = reinterpret_cast<floatx4*>(buf + (idx >> 5) * LDM + SOFF + ((idx & 31) << 2));
+    *q = *q + hv[it];
+  }
+}
+
 // Work item idx of the first inverse product: (row tile tm, K chunk s), enumerated from the bottom row tile up.
 // Chunk s of row tile tm is written 128*s columns to the right of chunk 0; the second product adds the chunks
 // while it loads its B operand (a fixed order, and no fence or atomic between workgroups: a device-scope fence
@@ -376,11 +449,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
   float* buf = reinterpret_cast<float*>(smem);
   using namespace gemmf32;
   const int bid = blockIdx.x;
+  // The workgroup on the dependence chain and the deep (K = 512) tiles of the inverse decide how long the launch
+  // takes; each shares its CU with a stream of short K = 128 tiles.  Wave priority lets them have the matrix pipes
+  // first: the short tiles lose what the long ones gain, the launch ends earlier.
+  if (bid <= inv_tiles) __builtin_amdgcn_s_setprio(3);
   if (bid == 0) {
-    const int t = i1 / NB - 1;  // last tile of the column-major upper-triangle order
+    // (the last tile of the trailing update's upper-triangle order: the other workgroups cover total-1 tiles)
     // the whole tile goes to the S position: what lies left of a row's diagonal lands in that row's Xt or unused
     // columns, and the Xt part is cleared next
-    tile_body<true, true, true>(g, t, t, 0, buf, 1, 1, [&](int r, int c, float v) { Sv(buf, r, c) = v; });
+    diag_tile_update(buf, A, ld, i1);
     __syncthreads();
     // Xt starts at zero in its 32x32 tiles below the diagonal ones (those are written whole by the elimination)
     for (int idx = threadIdx.x; idx < (NB - SB) * (NB / 4); idx += 256) {
@@ -455,11 +532,13 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
   }
   if ((ld & 3) || ((uintptr_t)A & 15)) return MQ_ERR_ARG;  // float4 access to rows of A
   int rc;
+  auto kc_of = [&](int) { return INV_KC; };  // one depth for all block rows: 2, 3 for the short rows measured no faster
   // the two products of block row b of the inverse (w = columns to the right of b)
   auto inv_first = [&](int b, int& tiles) {  // T^T (w x 128) = U22^T (w x w) * R12^T (w x 128), in K chunks
     const long p = (long)b * NB;
     const int w = C - (int)p - NB;
-    tiles = (w / NB) * ((w / NB + INV_KC - 1) / INV_KC);
+    const int kc = kc_of(w);
+    tiles = (w / NB) * ((w / NB + kc - 1) / kc);
     return GemmF32{A + (p + NB) * ld + (p + NB), A + p * ld + (p + NB), A + (p + NB) * ld + p, 1, ld, 1, ld, ld,
                    w, NB, w, 1.f, 0.f, 0, 1, 1, 0, 0, 0};
   };
@@ -468,7 +547,7 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
     const int w = C - (int)p - NB;
     tiles = w / NB;
     return GemmF32{A + p * ld + p, A + (p + NB) * ld + p, A + p * ld + (p + NB), ld, 1, 1, ld, ld,
-                   NB, w, NB, -1.f, 0.f, 0, 0, 1, 0, 0, 0, (w / NB + INV_KC - 1) / INV_KC, INV_KC, NB};
+                   NB, w, NB, -1.f, 0.f, 0, 0, 1, 0, 0, 0, (w / NB + kc_of(w) - 1) / kc_of(w), kc_of(w), NB};
   };
   const int B = C / NB;
   hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, A, ld, C - NB, info);
@@ -488,7 +567,8 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
     int t1 = 0;
     GemmF32 g1 = trail;
     if (b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
-    hipLaunchKernelGGL(trail_diag_kernel, dim3(total + t1), dim3(256), FUSED_SMEM, st, trail, total, g1, t1, INV_KC, A, ld,
+    hipLaunchKernelGGL(trail_diag_kernel, dim3(total + t1), dim3(256), FUSED_SMEM, st, trail, total, g1, t1,
+                       kc_of(C - i1 - NB), A, ld,
                        i1, info);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
@@ -501,7 +581,7 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
   if (B >= 2) {
     int t;
     GemmF32 g1 = inv_first(0, t);
-    hipLaunchKernelGGL(inv_first_kernel, dim3(t), dim3(256), gemmf32::SMEM_BYTES, st, g1, INV_KC);
+    hipLaunchKernelGGL(inv_first_kernel, dim3(t), dim3(256), gemmf32::SMEM_BYTES, st, g1, kc_of(C - NB));
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 g2 = inv_second(0, t);
     if ((rc = mq_launch_gemm_f32(g2, st)) != MQ_OK) return rc;
