@@ -128,14 +128,19 @@ class GPTQ:
     # ---- Hessian accumulation: src/gptq.py:73-105 ---------------------------------------------------
     @torch.no_grad()
     def update(self, input: Tensor) -> None:
-        if self.H is None:
-            self.H = torch.zeros((self.d_col, self.d_col), device=input.device, dtype=torch.float32)
         input = input.reshape(-1, input.shape[-1])
         if input.dtype != torch.bfloat16:
             raise TypeError(f"GPTQ.update needs bf16 activations, got {input.dtype}")
         num_new_samples = input.shape[0]
         if num_new_samples == 0:
+            if self.H is None:
+                self.H = torch.zeros((self.d_col, self.d_col), device=input.device, dtype=torch.float32)
             return  # the reference would divide 0/0 here when nothing was collected before
+        if self.H is None:
+            # the first product runs with beta = 0 and writes the whole upper triangle, the pre-step mirrors it:
+            # no need to clear 4*C^2 bytes first
+            alloc = torch.empty if self.num_samples == 0 else torch.zeros
+            self.H = alloc((self.d_col, self.d_col), device=input.device, dtype=torch.float32)
         beta = self.num_samples / (self.num_samples + num_new_samples)
         alpha = 2.0 / (self.num_samples + num_new_samples)
         # only the upper triangle is accumulated; quantization_pre_step mirrors it once
@@ -159,7 +164,8 @@ class GPTQ:
             if x.shape[0] == 0:
                 continue
             if h.H is None:
-                h.H = torch.zeros((h.d_col, h.d_col), device=x.device, dtype=torch.float32)
+                alloc = torch.empty if h.num_samples == 0 else torch.zeros  # beta = 0 below: nothing to clear
+                h.H = alloc((h.d_col, h.d_col), device=x.device, dtype=torch.float32)
             n = x.shape[0]
             Hs.append(h.H)
             Xs.append(x)
