@@ -98,6 +98,12 @@ int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_dtype, long 
  *          the device so that the caller need not read info back before queueing the loop.
  */
 int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream);
+/* The same with the input left untouched, as the torch calls it replaces leave self.H (src/gptq.py:236-242 build
+ * H_inv_cho in new tensors): H (upper triangle read, pitch ldh) -> U in A (pitch lda), A != H, A's contents on
+ * entry irrelevant.  The first elimination step reads from H what later steps find in A, so no copy is made.
+ */
+int mq_factor_upper_inverse_from(const float* H, long ldh, float* A, long lda, int C, int normalize, int* info,
+                                 void* stream);
 
 /* ---- (3) quantization grid and column loop ---------------------------------------------------------
  * Symmetric per-group scales.  Replaces find_quantization_meta (symmetric branch) as called from

@@ -24,6 +24,7 @@ SIGNATURES = {
     "mq_hessian_damp_workspace_bytes": (_sz, [_i]),
     "mq_hessian_damp": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp, _sz, _vp]),
     "mq_factor_upper_inverse": (_i, [_vp, _l, _i, _i, _vp, _vp]),
+    "mq_factor_upper_inverse_from": (_i, [_vp, _l, _vp, _l, _i, _i, _vp, _vp]),
     "mq_quant_grid_sym": (_i, [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "mq_mse_scale_sym": (_i, [_vp, _i, _l, _i, _i, _i, _vp, _vp, _i, _f, _f, _f, _i, _vp, _vp, _vp]),
     "mq_prepare_wt": (_i, [_vp, _i, _l, _i, _i, _vp, _vp, _vp, _l, _vp]),

@@ -53,6 +53,9 @@ struct GemmF32 {
   // column tile tn adds the first min(bsum, tn / bsum_c + 1) of them (0 = plain B).  Interior tiles only.
   int bsum, bsum_c;
   long bsum_stride;
+  // optional: the old C (the beta term) is read from another array of row pitch ldcs (nullptr = from C)
+  const float* Csrc;
+  long ldcs;
 };
 int mq_launch_gemm_f32(const GemmF32& g, hipStream_t stream);
 bool mq_gemm_operand_aligned(const float* p, long ld, long batch);

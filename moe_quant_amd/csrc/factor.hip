@@ -254,7 +254,7 @@ __device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, 
 // gidx0: global index of its first row.  preloaded: the caller already filled Sv (upper) and zeroed the 32x32 Xt
 // tiles below the diagonal ones (a barrier here orders those writes).  blk rows must be 16-byte aligned.
 __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info,
-                                                  bool preloaded) {
+                                                  bool preloaded, const float* src = nullptr, long src_ld = 0) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int idx = tid; idx < SB * LDI; idx += 256) buf[NB * LDM + idx] = (idx / LDI == idx % LDI) ? 1.f : 0.f;
   if (preloaded) __syncthreads();
@@ -263,7 +263,7 @@ __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long l
 #pragma unroll
     for (int it = 0; it < 16; ++it) {
       const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
-      v[it] = *reinterpret_cast<const float4*>(blk + (long)r * ld + c);
+      v[it] = *reinterpret_cast<const float4*>(src + (long)r * src_ld + c);
     }
 #pragma unroll
     for (int it = 0; it < 16; ++it) {
@@ -331,9 +331,11 @@ __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long l
   }
 }
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void revchol_diag_kernel(float* A, long ld, int i1, int* info) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void revchol_diag_kernel(const float* S, long lds,
+                                                                                                    float* A, long ld, int i1,
+                                                                                                    int* info) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false);
+  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false, S + (long)i1 * lds + i1, lds);
 }
 
 // The next diagonal tile, brought up to date by one workgroup on its own:  S(r,c) = H(r,c) - sum_k P(r,k) P(c,k)
@@ -343,10 +345,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void r
 // formed, dealt 3/3/2/2 to the four wavefronts (12k instead of 16k matrix-core cycles), operands and results
 // move 16 bytes at a time (transposed accumulators, as in tile_update), and the old tile is added row-wise from
 // registers loaded at the very start.  The result lands in the S position of buf; left of a row's diagonal is junk.
-__device__ __forceinline__ void diag_tile_update(float* buf, const float* A, long ld, int i1) {
+__device__ __forceinline__ void diag_tile_update(float* buf, const float* A, long ld, int i1, const float* Hsrc, long ldh) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const float* P = A + (long)(i1 - NB) * ld + i1;
-  const float* H = A + (long)(i1 - NB) * ld + (i1 - NB);
+  const float* H = Hsrc + (long)(i1 - NB) * ldh + (i1 - NB);  // the old tile: A itself, or the caller's matrix at the first step
   floatx4 pv[16], hv[16];
 #pragma unroll
   for (int it = 0; it < 16; ++it) {
@@ -356,7 +358,7 @@ __device__ __forceinline__ void diag_tile_update(float* buf, const float* A, lon
 #pragma unroll
   for (int it = 0; it < 16; ++it) {
     const int idx = tid + it * 256;
-    hv[it] = *reinterpret_cast<const floatx4*>(H + (long)(idx >> 5) * ld + ((idx & 31) << 2));
+    hv[it] = *reinterpret_cast<const floatx4*>(H + (long)(idx >> 5) * ldh + ((idx & 31) << 2));
   }
 #pragma unroll
   for (int it = 0; it < 16; ++it) {
@@ -457,7 +459,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
     // (the last tile of the trailing update's upper-triangle order: the other workgroups cover total-1 tiles)
     // the whole tile goes to the S position: what lies left of a row's diagonal lands in that row's Xt or unused
     // columns, and the Xt part is cleared next
-    diag_tile_update(buf, A, ld, i1);
+    diag_tile_update(buf, A, ld, i1, g.Csrc ? g.Csrc : A, g.Csrc ? g.ldcs : ld);
     __syncthreads();
     // Xt starts at zero in its 32x32 tiles below the diagonal ones (those are written whole by the elimination)
     for (int idx = threadIdx.x; idx < (NB - SB) * (NB / 4); idx += 256) {
@@ -513,8 +515,9 @@ constexpr size_t FUSED_SMEM = DIAG_SMEM > gemmf32::SMEM_BYTES ? DIAG_SMEM : gemm
 
 }  // namespace
 
-extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream) {
-  if (!A || !info || C <= 0 || ld < C) return MQ_ERR_ARG;
+// S: the matrix to factor (upper triangle read), A: where the factor is built and left.  S == A: in place.
+static int factor_impl(const float* S, long lds, float* A, long ld, int C, int normalize, int* info, void* stream) {
+  if (!S || !A || !info || C <= 0 || ld < C || lds < C) return MQ_ERR_ARG;
   if (C % NB != 0) return MQ_ERR_ARG;  // the host pads with an identity block
   hipStream_t st = (hipStream_t)stream;
   static bool attr_done = false;
@@ -530,7 +533,7 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
                               (int)gemmf32::SMEM_BYTES);
     attr_done = true;
   }
-  if ((ld & 3) || ((uintptr_t)A & 15)) return MQ_ERR_ARG;  // float4 access to rows of A
+  if ((ld & 3) || ((uintptr_t)A & 15) || (lds & 3) || ((uintptr_t)S & 15)) return MQ_ERR_ARG;  // float4 access to rows
   int rc;
   auto kc_of = [&](int) { return INV_KC; };  // one depth for all block rows: 2, 3 for the short rows measured no faster
   // the two products of block row b of the inverse (w = columns to the right of b)
@@ -550,19 +553,25 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
                    NB, w, NB, -1.f, 0.f, 0, 0, 1, 0, 0, 0, (w / NB + kc_of(w) - 1) / kc_of(w), kc_of(w), NB};
   };
   const int B = C / NB;
-  hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, A, ld, C - NB, info);
+  hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, S, lds, A, ld, C - NB, info);
   if ((rc = mq_check_launch()) != MQ_OK) return rc;
   for (int b = B - 1; b >= 1; --b) {
     const int i1 = b * NB;
     float* P = A + i1;  // panel: rows [0,i1), cols [i1, i1+NB)
     const float* Dinv = A + (long)i1 * ld + i1;
-    GemmF32 panel{P, Dinv, P, ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
+    // the first step reads what no earlier step has touched: from S (every later read finds its data in A)
+    const bool first = (b == B - 1) && (S != A);
+    GemmF32 panel{first ? S + i1 : P, Dinv, P, first ? lds : ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
     int t2 = 0;
     GemmF32 g2 = panel;
     if (b + 1 <= B - 2) g2 = inv_second(b + 1, t2);  // row b+1: its T was produced in the previous launch
     hipLaunchKernelGGL(panel_inv_kernel, dim3(b + t2), dim3(256), gemmf32::SMEM_BYTES, st, panel, b, g2, t2);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
+    if (first) {
+      trail.Csrc = S;
+      trail.ldcs = lds;
+    }
     const int tiles = i1 / NB, total = tiles * (tiles + 1) / 2;
     int t1 = 0;
     GemmF32 g1 = trail;
@@ -588,4 +597,14 @@ extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, 
   }
   hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize, info);
   return mq_check_launch();
+}
+
+extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream) {
+  return factor_impl(A, ld, A, ld, C, normalize, info, stream);
+}
+
+extern "C" int mq_factor_upper_inverse_from(const float* H, long ldh, float* A, long lda, int C, int normalize, int* info,
+                                            void* stream) {
+  if (H == A) return MQ_ERR_ARG;
+  return factor_impl(H, ldh, A, lda, C, normalize, info, stream);
 }

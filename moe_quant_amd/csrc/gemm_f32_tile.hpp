@@ -178,6 +178,8 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
       lb.load(B, g.sbn, g.sbk, n0, g.N, (k0), ke, vecB, tid);   \
     }                                                           \
   } while (0)
+  const float* Cold = g.Csrc ? g.Csrc + (C - g.C) : C;  // where the beta term is read from
+  const long ldcold = g.Csrc ? g.ldcs : g.ldc;
   const int nk = (ke - kb + BK - 1) / BK;
   if (nk > 0) MQ_GEMM_FETCH(kb);
   // Interior tiles that go to memory move C sixteen bytes at a time, row-wise (a wavefront covers two rows of 512
@@ -192,7 +194,7 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
 #pragma unroll
       for (int it = 0; it < 16; ++it) {
         const int idx = tid + it * 256;
-        cold4[it] = *reinterpret_cast<const floatx4*>(C + (long)(m0 + (idx >> 5)) * g.ldc + n0 + ((idx & 31) << 2));
+        cold4[it] = *reinterpret_cast<const floatx4*>(Cold + (long)(m0 + (idx >> 5)) * ldcold + n0 + ((idx & 31) << 2));
       }
     }
   } else if (beta != 0.f) {
@@ -204,7 +206,7 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-          if (FAST || (row < g.M && col < g.N)) cold[i][j][v] = C[(long)row * g.ldc + col];
+          if (FAST || (row < g.M && col < g.N)) cold[i][j][v] = Cold[(long)row * ldcold + col];
         }
       }
   }
@@ -301,7 +303,8 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   int kb = 0, ke = g.K;
   if (g.ktrim == 1) ke = min(g.K, m0 + BM);
   if (g.ktrim == 2) kb = m0;
-  const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0);  // C moves 16 bytes at a time
+  const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0 &&  // C moves 16 bytes at a time
+                                 (!g.Csrc || ((((uintptr_t)g.Csrc) & 15) == 0 && (g.ldcs & 3) == 0)));
   const bool interior = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N && ((ke - kb) % BK == 0);
   if (interior) tile_core<A_KC, B_KC, true, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
   else tile_core<A_KC, B_KC, false, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);

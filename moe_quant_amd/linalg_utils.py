@@ -26,6 +26,9 @@ def inverse_cholesky_factor(H: Tensor, normalize: bool = True):
     GPTQ._get_hessian_inverse returns, src/gptq.py:236-242).  H is not modified.
     Returns (U, info): info is a device int32 tensor, 0 on success, else the 1-based pivot that failed."""
     C = H.shape[0]
+    if (C % 128 == 0 and H.dtype == torch.float32 and H.stride(1) == 1 and H.stride(0) % 4 == 0
+            and H.data_ptr() % 16 == 0):
+        return ops.factor_upper_inverse_from(H, normalize=normalize)  # reads H in place of a copy of it
     A = _padded_copy(H)
     info = ops.factor_upper_inverse_(A, normalize=normalize)
     U = A if A.shape[0] == C else A[:C, :C].contiguous()

@@ -172,6 +172,22 @@ def factor_upper_inverse_(A: Tensor, info: Optional[Tensor] = None, normalize: b
     return info
 
 
+def factor_upper_inverse_from(H: Tensor, info: Optional[Tensor] = None, normalize: bool = True):
+    """Like factor_upper_inverse_ but H is left untouched: returns (U, info) with U a new tensor."""
+    _dev(H, info)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1 or C % 128:
+        raise ValueError("H must be (C,C) fp32, unit column stride, C % 128 == 0")
+    if info is None:
+        info = torch.zeros(1, dtype=torch.int32, device=H.device)
+    U = torch.empty((C, C), dtype=torch.float32, device=H.device)
+    rc = lib.mq_factor_upper_inverse_from(H.data_ptr(), H.stride(0), U.data_ptr(), U.stride(0), C, int(normalize),
+                                          info.data_ptr(), _stream(H))
+    check(rc, "mq_factor_upper_inverse_from")
+    return U, info
+
+
 # ---- (3) grid, layout, loop --------------------------------------------------------------------------
 def quant_grid_sym(W: Tensor, group_size: int, bits: int, round_dtype, dead_cols: Optional[Tensor] = None,
                    want_transposed: bool = True) -> Tuple[Tensor, Optional[Tensor]]:

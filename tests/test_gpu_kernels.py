@@ -162,6 +162,27 @@ def test_factor_vs_torch_chain(dev, C):
     assert rel < max(5e-6, 5 * rel32)
 
 
+@pytest.mark.parametrize("C", [128, 256, 1024])
+def test_factor_from_equals_in_place(dev, C):
+    """The entry point that leaves H untouched builds the same bits as the in-place one, on a destination full of NaN."""
+    _say(f"factor_from C={C}")
+    H = _spd(C, seed=17).to(dev)
+    H0 = H.clone()
+    A = H.clone()
+    info_a = ops.factor_upper_inverse_(A)
+    lib = __import__("moe_quant_amd._lib", fromlist=["load"]).load()
+    U = torch.full((C, C), float("nan"), device=dev)
+    info_u = torch.zeros(1, dtype=torch.int32, device=dev)
+    rc = lib.mq_factor_upper_inverse_from(H.data_ptr(), H.stride(0), U.data_ptr(), U.stride(0), C, 1, info_u.data_ptr(),
+                                          None)
+    torch.cuda.synchronize()
+    assert rc == 0 and int(info_a.item()) == 0 and int(info_u.item()) == 0
+    assert torch.equal(H, H0)
+    assert torch.equal(U, A)
+    # H == A is refused
+    assert lib.mq_factor_upper_inverse_from(H.data_ptr(), C, H.data_ptr(), C, C, 1, info_u.data_ptr(), None) != 0
+
+
 def test_factor_reports_non_pd(dev):
     C = 256
     H = _spd(C, 77)
