@@ -68,6 +68,16 @@ __device__ __forceinline__ float round_sel(float x, int rd) {
   return rd == DT_BF16 ? b : (rd == DT_F16 ? h : x);
 }
 
+// rounding to the scale/weight dtype known at compile time (RD: 0 fp32, 1 bf16, 2 fp16); the hardware bf16
+// conversion rounds to nearest even like round_to_bf16
+template <int RD>
+__device__ __forceinline__ float round_rd(float x) {
+  if (RD == DT_BF16) return (float)(__bf16)x;
+  if (RD == DT_F16) return __half2float(__float2half_rn(x));
+  return x;
+}
+
+template <int RD>
 __global__ __launch_bounds__(256) void mse_scale_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C, int g,
                                                         int G, const uint8_t* __restrict__ dead, const float* __restrict__ p,
                                                         int P, float qzero, float maxq, float norm, int rd,
@@ -77,11 +87,15 @@ __global__ __launch_bounds__(256) void mse_scale_kernel(const void* __restrict__
   if (item >= (long)R * G) return;
   const int row = (int)(item / G), grp = (int)(item - (long)row * G);
   const float s0 = scale_rg[(long)row * G + grp];
-  float sp[MSE_NC], loss[MSE_NC];
+  // x / s with IEEE rounding from a reciprocal computed once per candidate: q0 = RN(x*rcp), q1 = RN(q0 +
+  // (x - q0*s)*rcp) is the correctly rounded quotient when rcp = RN(1/s) (Markstein); infinities and NaNs keep q0,
+  // which is what the division gives there
+  float sp[MSE_NC], rcp[MSE_NC], loss[MSE_NC];
 #pragma unroll
   for (int c = 0; c < MSE_NC; ++c) {
     const int idx = lane + 64 * c;
     sp[c] = round_sel(s0 * p[min(idx, P - 1)], rd);
+    rcp[c] = 1.0f / sp[c];
     loss[c] = 0.f;
   }
   const int c0 = grp * g;
@@ -99,9 +113,11 @@ __global__ __launch_bounds__(256) void mse_scale_kernel(const void* __restrict__
 #pragma unroll
       for (int c = 0; c < MSE_NC; ++c) {
         if (64 * c < P) {  // wave-uniform
-          float q = floorf(x / sp[c] + qzero + 0.5f);
+          const float q0 = x * rcp[c];
+          const float q1 = fmaf(fmaf(-q0, sp[c], x), rcp[c], q0);
+          float q = floorf((fabsf(q0) < 3.0e38f ? q1 : q0) + qzero + 0.5f);
           q = fminf(fmaxf(q, 0.f), maxq);
-          const float d = fabsf(round_sel((q - qzero) * sp[c], rd) - x);
+          const float d = fabsf(round_rd<RD>((q - qzero) * sp[c]) - x);
           loss[c] += __builtin_amdgcn_exp2f(norm * __builtin_amdgcn_logf(d));
         }
       }
@@ -337,8 +353,14 @@ extern "C" int mq_mse_scale_sym(const void* W, int w_dtype, long ldw, int R, int
   if (P <= 0 || P > 64 * MSE_NC) return MQ_ERR_ARG;
   const int G = C / group_size;
   const long items = (long)R * G;
-  hipLaunchKernelGGL(mse_scale_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, W, w_dtype, ldw,
-                     R, C, group_size, G, dead_cols, p, P, qzero, maxq, norm, round_dtype, scale_rg, scale_gr);
+  const dim3 grid((unsigned)((items + 3) / 4));
+#define MQ_MSE(RD_)                                                                                                   \
+  hipLaunchKernelGGL(mse_scale_kernel<RD_>, grid, dim3(256), 0, (hipStream_t)stream, W, w_dtype, ldw, R, C, group_size, G, \
+                     dead_cols, p, P, qzero, maxq, norm, round_dtype, scale_rg, scale_gr)
+  if (round_dtype == DT_BF16) MQ_MSE(DT_BF16);
+  else if (round_dtype == DT_F16) MQ_MSE(DT_F16);
+  else MQ_MSE(0);
+#undef MQ_MSE
   return mq_check_launch();
 }
 
