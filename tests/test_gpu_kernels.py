@@ -306,6 +306,22 @@ def test_grid_bit_exact(dev, dtype, g):
     assert torch.equal(s_gr.cpu(), s_ref.t())
 
 
+@pytest.mark.parametrize("g", [32, 128, 512])
+def test_grid_wide_rows_and_dead_columns(dev, g):
+    """Rows wider than one wavefront pass of the 16-byte kernel (2048 columns), ragged last pass, dead columns."""
+    R, C = 40, 2048 + 1536
+    W = _rand((R, C), 21, 0.02).bfloat16()
+    dead = torch.zeros(C, dtype=torch.uint8)
+    dead[[0, 5, 2047, 2048, C - 1]] = 1
+    dead[1024:1024 + g] = 1  # a whole group dead -> bf16(1e-12)
+    Wm = W.float().clone()
+    Wm[:, dead.bool()] = 0
+    s_ref, _, _ = O.quantization_grid(Wm, g, 4, torch.bfloat16)
+    s_rg, s_gr = ops.quant_grid_sym(W.to(dev), g, 4, torch.bfloat16, dead_cols=dead.to(dev))
+    assert torch.equal(s_rg.cpu(), s_ref)
+    assert torch.equal(s_gr.cpu(), s_ref.t())
+
+
 def test_prepare_and_untranspose(dev):
     R, C = 200, 320
     W = _rand((R, C), 12, 0.02).bfloat16()
