@@ -131,15 +131,17 @@ __global__ __launch_bounds__(256) void wcol_scan_kernel(const void* __restrict__
 
 // One workgroup: dead[c] = pruned[c] || no strip saw a nonzero weight; damp = rel_damp * mean(diag after the
 // fix); sums run in a fixed order (thread-strided partials, then a tree), so the result is reproducible.
-__global__ __launch_bounds__(256) void damp_scalar_kernel(const float* __restrict__ H, long ldh, int C,
-                                                          const uint8_t* __restrict__ pruned,
-                                                          const uint8_t* __restrict__ nonzero, float rel_damp,
-                                                          uint8_t* __restrict__ dead, float* __restrict__ damp_out, int* flags) {
-  __shared__ float ssum[256];
-  __shared__ int scnt[256];
+__global__ __launch_bounds__(1024) void damp_scalar_kernel(const float* __restrict__ H, long ldh, int C,
+                                                           const uint8_t* __restrict__ pruned,
+                                                           const uint8_t* __restrict__ nonzero, float rel_damp,
+                                                           uint8_t* __restrict__ dead, float* __restrict__ damp_out, int* flags) {
+  __shared__ float ssum[1024];
+  __shared__ int scnt[1024];
   float s = 0.f;
   int n = 0;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  // (1024 threads and an unrolled loop: every diagonal element is its own cache line, the loads must overlap)
+#pragma unroll 4
+  for (int c = threadIdx.x; c < C; c += 1024) {
     uint32_t nz = 0;
 #pragma unroll
     for (int q = 0; q < STRIPS; ++q) nz |= nonzero[(long)q * C + c];
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(256) void damp_scalar_kernel(const float* __restric
   ssum[threadIdx.x] = s;
   scnt[threadIdx.x] = n;
   __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
+  for (int w = 512; w > 0; w >>= 1) {
     if (threadIdx.x < w) {
       ssum[threadIdx.x] += ssum[threadIdx.x + w];
       scnt[threadIdx.x] += scnt[threadIdx.x + w];
@@ -219,7 +221,7 @@ extern "C" int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_d
                        nonzero);
   }
   // the strips are laid out with pitch C (not the padded c) inside the first STRIPS*c bytes
-  hipLaunchKernelGGL(damp_scalar_kernel, dim3(1), dim3(256), 0, st, H, ldh, C, pruned, nonzero, rel_damp, dead, damp, flags);
+  hipLaunchKernelGGL(damp_scalar_kernel, dim3(1), dim3(1024), 0, st, H, ldh, C, pruned, nonzero, rel_damp, dead, damp, flags);
   hipLaunchKernelGGL(damp_apply_kernel, dim3(C), dim3(256), 0, st, H, ldh, C, dead, damp, flags);
   return mq_check_launch();
 }
