@@ -404,6 +404,37 @@ def test_loop_quantizer_arithmetic_is_ieee_exact(dev):
     assert torch.equal(Wd.cpu(), ((want - 8.0) * s).bfloat16().float())
 
 
+@pytest.mark.parametrize("rd", [torch.bfloat16, torch.float16, torch.float32])
+def test_loop_block_wide_scale_row_is_ieee_exact(dev, rd):
+    """Grouped scales whose group covers a whole block: the kernel divides through a reciprocal computed once per
+    block (q0 = x*rcp, q1 = fma(fma(-q0, s, x), rcp, q0)).  With U = I, 2M (w, s) pairs incl. zero, tiny and huge
+    scales must give exactly floor(w / s + 8.5) with IEEE division, and the dequantized weights the rounded (q-8)*s."""
+    R, C, gsz = 2048, 1024, 128
+    g = torch.Generator().manual_seed(123)
+    W = torch.randn(R, C, generator=g) * 0.02
+    W[:, 100] = 0.0
+    W[5, :] = torch.linspace(-0.2, 0.2, C)
+    G = C // gsz
+    s = (torch.rand(G, R, generator=g) * 0.02 + 1e-4).bfloat16().float()
+    s[1, :512] = torch.tensor(1e-12).bfloat16().float()   # the all-zero-group scale
+    s[2, :512] = 0.0                                       # division by zero: +-inf and NaN quotients
+    s[3, :512] = 3.0e-39                                   # a denormal scale: its reciprocal overflows
+    s[4] = (W[:, 4 * gsz:5 * gsz].abs().amax(1) / 7.5 + 1e-12).bfloat16().float()  # many .5 boundaries
+    s[5, :512] = 1e30                                      # tiny quotients
+    srow = (torch.arange(C) // gsz).to(torch.int32)
+    Wt = W.t().contiguous()
+    s_rep = s[srow.long()]                                 # (C, R)
+    want = torch.floor(Wt / s_rep + 8.0 + 0.5)
+    want = torch.where(torch.isnan(want), torch.zeros_like(want), want).clamp(0, 15)  # fmax(NaN, 0) = 0
+    Wd = Wt.clone().to(dev)
+    Qt = ops.gptq_loop_(Wd, torch.eye(C, device=dev), s.to(dev), srow.to(dev), None, 8.0, 15.0, rd, 128)
+    assert torch.equal(Qt.cpu().float(), want)
+    deq = ((want - 8.0) * s_rep).to(rd).float()
+    got = Wd.cpu()
+    ok = torch.isfinite(deq)
+    assert torch.equal(got[ok], deq[ok])
+
+
 def test_loop_compact_scale_and_perm(dev):
     R, C, g = 128, 512, 64
     W32, U, s, s_rep, z_rep, maxq, perm, perm_inv = _loop_case(R, C, 8, g=g, act_order=True)
