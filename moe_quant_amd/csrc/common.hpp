@@ -56,6 +56,8 @@ struct GemmF32 {
   // optional: the old C (the beta term) is read from another array of row pitch ldcs (nullptr = from C)
   const float* Csrc;
   long ldcs;
+  // 1: interior tiles too run on the fp32 matrix cores (default: operands split into bf16 pieces, bf16 cores)
+  int fp32_mfma;
 };
 int mq_launch_gemm_f32(const GemmF32& g, hipStream_t stream);
 bool mq_gemm_operand_aligned(const float* p, long ld, long batch);

@@ -285,6 +285,190 @@ __device__ __forceinline__ void tile_core(const GemmF32& g, int m0, int n0, int 
 #undef MQ_GEMM_FETCH
 }
 
+// =============================================================================================
+// Interior tiles on the bf16 matrix cores.  Every fp32 operand element is split into three bf16 pieces,
+// x = hi + mid + lo (hi = RN(x), mid = RN(x - hi), lo = RN(x - hi - mid); 24 significand bits in all), and the
+// product is formed from the six piece products that matter, hi*hi + hi*mid + mid*hi + hi*lo + lo*hi + mid*mid,
+// each exact in the fp32 accumulator of v_mfma_f32_32x32x16_bf16 (what is dropped is below 2^-23 of |a||b|).
+// The bf16 pipe runs 16 times the fp32 one, so six products cost 0.4 of the fp32 MFMA time; against an fp64
+// product the result is as close as the fp32 MFMA path's (1.6e-7 vs 2.0e-7 relative on random 512x512x128).
+// BK = 16 per stage.  LDS per operand and stage, three planes:
+//   k-contiguous operand : [k/8][x][8]   bf16, 4 KB a plane: a lane's MFMA fragment (8 k of one row) is one b128 read,
+//                          lanes 0..31 read 512 contiguous bytes;
+//   x-contiguous operand : [k][x] bf16 with 288-byte rows, 4.5 KB a plane: fragments come out of the transposing
+//                          read ds_read_b64_tr_b16 (16 lanes fetch a 4 k x 16 x patch, each ends up with 4 k of its x).
+// =============================================================================================
+namespace split {
+constexpr int SBK = 16;
+constexpr int KPLANE = 4096, XROW = 288, XPLANE = SBK * XROW;
+constexpr int OPB_MAX = 3 * XPLANE;
+constexpr int STAGEB = 2 * OPB_MAX;
+static_assert(2 * STAGEB <= (int)SMEM_BYTES, "two stages must fit in the fp32 core's LDS");
+typedef __bf16 bf16x4v __attribute__((ext_vector_type(4)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+template <bool KC>
+struct Loader {
+  floatx4 r[2];
+  // element (x, k) at p[x*sx + k*sk]; KC: sk == 1, else sx == 1
+  __device__ __forceinline__ const float* addr(const float* p, long sx, long sk, int x0, int k0, int it, int tid) const {
+    const int idx = tid + it * 256;
+    if (KC) return p + (long)(x0 + (idx >> 2)) * sx + k0 + ((idx & 3) << 2);
+    return p + (long)(k0 + (idx >> 5)) * sk + x0 + ((idx & 31) << 2);
+  }
+  __device__ __forceinline__ void load(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) r[it] = *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
+  }
+  __device__ __forceinline__ void add(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) r[it] += *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
+  }
+  __device__ __forceinline__ void store(unsigned char* op, int tid) const {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int idx = tid + it * 256;
+      const floatx4 v = r[it];
+      const bf16x4v hi = __builtin_convertvector(v, bf16x4v);
+      const floatx4 r1 = v - __builtin_convertvector(hi, floatx4);
+      const bf16x4v mid = __builtin_convertvector(r1, bf16x4v);
+      const floatx4 r2 = r1 - __builtin_convertvector(mid, floatx4);
+      const bf16x4v lo = __builtin_convertvector(r2, bf16x4v);
+      unsigned char* q;
+      int plane;
+      if (KC) {
+        const int x = idx >> 2, k4 = (idx & 3) << 2;
+        q = op + (k4 >> 3) * 2048 + x * 16 + (k4 & 7) * 2;
+        plane = KPLANE;
+      } else {
+        const int k = idx >> 5, x4 = (idx & 31) << 2;
+        q = op + k * XROW + x4 * 2;
+        plane = XPLANE;
+      }
+      *reinterpret_cast<bf16x4v*>(q) = hi;
+      *reinterpret_cast<bf16x4v*>(q + plane) = mid;
+      *reinterpret_cast<bf16x4v*>(q + 2 * plane) = lo;
+    }
+  }
+};
+
+// the three planes of the fragment of rows xt..xt+31 for this lane (row xt + lane%32, k = 8*(lane/32)..+7)
+template <bool KC>
+__device__ __forceinline__ void frag(const unsigned char* op, int xt, int lane, bf16x8n (&f)[3]) {
+  if (KC) {
+    const unsigned char* q = op + (lane >> 5) * 2048 + (xt + (lane & 31)) * 16;
+#pragma unroll
+    for (int p = 0; p < 3; ++p) f[p] = *reinterpret_cast<const bf16x8n*>(q + p * KPLANE);
+  } else {
+    const int L = lane & 15;
+    const unsigned char* q = op + (8 * (lane >> 5) + (L >> 2)) * XROW + (xt + 16 * ((lane >> 4) & 1) + 4 * (L & 3)) * 2;
+#pragma unroll
+    for (int p = 0; p < 3; ++p) {
+      const short4v a = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (short4v __attribute__((address_space(3)))*)(q + p * XPLANE));
+      const short4v b = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (short4v __attribute__((address_space(3)))*)(q + p * XPLANE + 4 * XROW));
+      f[p] = __builtin_bit_cast(bf16x8n, __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  }
+}
+}  // namespace split
+
+template <bool A_KC, bool B_KC>
+__device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0, int kb, int ke, const float* __restrict__ A,
+                                                const float* __restrict__ B, float* C, float* smem_f) {
+  using namespace split;
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_f);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, lr = lane & 31, lk = lane >> 5;
+  const float alpha = g.alpha, beta = g.beta;
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  Loader<A_KC> la;
+  Loader<B_KC> lb;
+  const int nsum = g.bsum ? min(g.bsum, (n0 / BN) / g.bsum_c + 1) : 1;  // arrays summed into the B operand
+#define MQ_SPLIT_FETCH(k0)                                                                     \
+  do {                                                                                         \
+    la.load(A, g.sam, g.sak, m0, (k0), tid);                                                   \
+    lb.load(B, g.sbn, g.sbk, n0, (k0), tid);                                                   \
+    for (int s_ = 1; s_ < nsum; ++s_) lb.add(B + s_ * g.bsum_stride, g.sbn, g.sbk, n0, (k0), tid); \
+  } while (0)
+  const float* Cold = g.Csrc ? g.Csrc + (C - g.C) : C;
+  const long ldcold = g.Csrc ? g.ldcs : g.ldc;
+  const int nk = (ke - kb) / SBK;
+  if (nk > 0) MQ_SPLIT_FETCH(kb);
+  constexpr int LDC_S = BN + 4;
+  floatx4 cold4[16];
+  if (beta != 0.f) {
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int idx = tid + it * 256;
+      cold4[it] = *reinterpret_cast<const floatx4*>(Cold + (long)(m0 + (idx >> 5)) * ldcold + n0 + ((idx & 31) << 2));
+    }
+  }
+  if (nk > 0) {
+    la.store(smem, tid);
+    lb.store(smem + OPB_MAX, tid);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) MQ_SPLIT_FETCH(kb + (kt + 1) * SBK);
+    const unsigned char* as = smem + cur * STAGEB;
+    const unsigned char* bs = as + OPB_MAX;
+    bf16x8n fa[2][3], fb[2][3];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      frag<A_KC>(as, wm * 64 + i * 32, lane, fa[i]);
+      frag<B_KC>(bs, wn * 64 + i * 32, lane, fb[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {  // small terms first
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][1], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][2], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][2], fb[j][0], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][1], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][0], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][0], acc[i][j], 0, 0, 0);
+      }
+    if (kt + 1 < nk) {
+      la.store(smem + (cur ^ 1) * STAGEB, tid);
+      lb.store(smem + (cur ^ 1) * STAGEB + OPB_MAX, tid);
+    }
+    __syncthreads();
+  }
+#undef MQ_SPLIT_FETCH
+  float* cs = smem_f;  // the loop's last barrier has passed: no wavefront reads operands any more
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        cs[(wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3)) * LDC_S + wn * 64 + j * 32 + lr] = acc[i][j][v];
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+    const floatx4 a4 = *reinterpret_cast<const floatx4*>(cs + r * LDC_S + c);
+    floatx4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float x = alpha * a4[e];
+      if (beta != 0.f) x = fmaf(beta, cold4[it][e], x);
+      o[e] = x;
+    }
+    *reinterpret_cast<floatx4*>(C + (long)(m0 + r) * g.ldc + n0 + c) = o;
+  }
+}
+
 // One 128x128 output tile (tm, tn) of problem g (batch index z).  smem: SMEM_BYTES of LDS.
 // The old C tile is fetched before the K loop (when beta != 0) so its latency hides behind the products;
 // it is added after the accumulation, never fed through the accumulator.
@@ -305,7 +489,12 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   if (g.ktrim == 2) kb = m0;
   const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0 &&  // C moves 16 bytes at a time
                                  (!g.Csrc || ((((uintptr_t)g.Csrc) & 15) == 0 && (g.ldcs & 3) == 0)));
-  const bool interior = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N && ((ke - kb) % BK == 0);
+  const bool inside = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N;
+  if (!LDS_OUT && !g.fp32_mfma && inside && ((ke - kb) % split::SBK == 0)) {
+    tile_core_split<A_KC, B_KC>(g, m0, n0, kb, ke, A, B, C, smem);
+    return;
+  }
+  const bool interior = inside && ((ke - kb) % BK == 0);
   if (interior) tile_core<A_KC, B_KC, true, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
   else tile_core<A_KC, B_KC, false, LDS_OUT, Sink>(g, m0, n0, kb, ke, A, B, C, smem, vecA, vecB, sink);
 }
