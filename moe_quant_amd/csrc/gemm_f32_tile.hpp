@@ -320,9 +320,25 @@ struct Loader {
 #pragma unroll
     for (int it = 0; it < 2; ++it) r[it] = *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
   }
-  __device__ __forceinline__ void add(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
+  // r += the same tile of `n` more arrays, `stride` elements apart; four arrays' loads are in flight together
+  __device__ __forceinline__ void add_many(const float* __restrict__ p, long stride, int n, long sx, long sk, int x0, int k0,
+                                           int tid) {
+    for (int s0 = 0; s0 < n; s0 += 4) {
+      floatx4 t[4][2];
 #pragma unroll
-    for (int it = 0; it < 2; ++it) r[it] += *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+          // (arrays past the last one re-read the last: the value is dropped below)
+          const float* q = addr(p + (long)min(s0 + u, n - 1) * stride, sx, sk, x0, k0, it, tid);
+          t[u][it] = *reinterpret_cast<const floatx4*>(q);
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int it = 0; it < 2; ++it)
+          if (s0 + u < n) r[it] += t[u][it];
+    }
   }
   __device__ __forceinline__ void store(unsigned char* op, int tid) const {
 #pragma unroll
@@ -396,7 +412,7 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
   do {                                                                                         \
     la.load(A, g.sam, g.sak, m0, (k0), tid);                                                   \
     lb.load(B, g.sbn, g.sbk, n0, (k0), tid);                                                   \
-    for (int s_ = 1; s_ < nsum; ++s_) lb.add(B + s_ * g.bsum_stride, g.sbn, g.sbk, n0, (k0), tid); \
+    if (nsum > 1) lb.add_many(B + g.bsum_stride, g.bsum_stride, nsum - 1, g.sbn, g.sbk, n0, (k0), tid); \
   } while (0)
   const float* Cold = g.Csrc ? g.Csrc + (C - g.C) : C;
   const long ldcold = g.Csrc ? g.ldcs : g.ldc;
@@ -427,17 +443,15 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
       frag<A_KC>(as, wm * 64 + i * 32, lane, fa[i]);
       frag<B_KC>(bs, wn * 64 + i * 32, lane, fb[i]);
     }
+    // small terms first; the four accumulators take turns, so consecutive instructions never depend on each other
+    constexpr int PA[6] = {1, 0, 2, 0, 1, 0}, PB[6] = {1, 2, 0, 1, 0, 0};
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int t = 0; t < 6; ++t)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {  // small terms first
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][1], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][2], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][2], fb[j][0], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][1], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][1], fb[j][0], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][0], fb[j][0], acc[i][j], 0, 0, 0);
-      }
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][PA[t]], fb[j][PB[t]], acc[i][j], 0, 0, 0);
     if (kt + 1 < nk) {
       la.store(smem + (cur ^ 1) * STAGEB, tid);
       lb.store(smem + (cur ^ 1) * STAGEB + OPB_MAX, tid);
