@@ -476,15 +476,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
   }
 }
 
-// Panel product of step b (P = H_ab Dinv^T, one tile per row block) together with the second product of the
-// inverse's block row b+1 (U12 = -U11 T, one tile per column block): two independent GEMMs in one launch.
+// Panel product of step b (P = H_ab Dinv^T, 128 columns wide, in place: tiles of 64 rows x all 128 columns)
+// together with the second product of the inverse's block row b+1 (U12 = -U11 T, 128 rows high: tiles of
+// 64 x 64): two independent GEMMs with K = 128 in one launch.
 __global__ __launch_bounds__(256) void panel_inv_kernel(GemmF32 gp, int panel_tiles, GemmF32 g2, int inv_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* buf = reinterpret_cast<float*>(smem);
-  using namespace gemmf32;
   const int bid = blockIdx.x;
-  if (bid < panel_tiles) tile_body<true, true>(gp, bid, 0, 0, buf, 1, 1);
-  else tile_body<true, true>(g2, 0, bid - panel_tiles, 0, buf, 1, 1);
+  if (bid < panel_tiles) {
+    gemmf32::tile_short<2>(gp, bid * 64, 0, buf);
+  } else {
+    const int r = bid - panel_tiles;
+    gemmf32::tile_short<1>(g2, (r & 1) * 64, (r >> 1) * 64, buf);
+  }
 }
 
 // U[j,k] <- U[j,k] / U[j,j] for k > j, 1 on the diagonal, 0 for k < j (normalize == 0: only the zeroing).
@@ -528,7 +532,7 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     (void)hipFuncSetAttribute((const void*)trail_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)FUSED_SMEM);
     (void)hipFuncSetAttribute((const void*)panel_inv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)gemmf32::SMEM_BYTES);
+                              (int)gemmf32::short_smem_bytes(2));
     (void)hipFuncSetAttribute((const void*)inv_first_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)gemmf32::SMEM_BYTES);
     attr_done = true;
@@ -565,7 +569,9 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     int t2 = 0;
     GemmF32 g2 = panel;
     if (b + 1 <= B - 2) g2 = inv_second(b + 1, t2);  // row b+1: its T was produced in the previous launch
-    hipLaunchKernelGGL(panel_inv_kernel, dim3(b + t2), dim3(256), gemmf32::SMEM_BYTES, st, panel, b, g2, t2);
+    static_assert(NB == gemmf32::SHORT_K, "the panel kernel's tiles take K = 128");
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(2 * b + 4 * t2), dim3(256), gemmf32::short_smem_bytes(2), st, panel, 2 * b,
+                       g2, 4 * t2);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     if (first) {

@@ -320,13 +320,14 @@ struct Loader {
 #pragma unroll
     for (int it = 0; it < 2; ++it) r[it] = *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
   }
-  // r += the same tile of `n` more arrays, `stride` elements apart; four arrays' loads are in flight together
+  // r += the same tile of `n` more arrays, `stride` elements apart; eight arrays' loads are in flight together
   __device__ __forceinline__ void add_many(const float* __restrict__ p, long stride, int n, long sx, long sk, int x0, int k0,
                                            int tid) {
-    for (int s0 = 0; s0 < n; s0 += 4) {
-      floatx4 t[4][2];
+    constexpr int NB8 = 8;
+    for (int s0 = 0; s0 < n; s0 += NB8) {
+      floatx4 t[NB8][2];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < NB8; ++u)
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
           // (arrays past the last one re-read the last: the value is dropped below)
@@ -334,7 +335,7 @@ struct Loader {
           t[u][it] = *reinterpret_cast<const floatx4*>(q);
         }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < NB8; ++u)
 #pragma unroll
         for (int it = 0; it < 2; ++it)
           if (s0 + u < n) r[it] += t[u][it];
@@ -480,6 +481,128 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
       o[e] = x;
     }
     *reinterpret_cast<floatx4*>(C + (long)(m0 + r) * g.ldc + n0 + c) = o;
+  }
+}
+
+// A 64 x (64 NH) output tile with K = 128, both operands K-contiguous, beta == 0: for launches of a few
+// short products, which are nothing but latency (the core above waits one memory round trip per 16 k, and
+// a 128x128 tile keeps one CU busy where several could share the work).  All of K is requested at once;
+// the arrays of a summed B operand are fetched eight at a time.  Operands pass through LDS in two halves of
+// 64 k (short_smem_bytes(NH)).  Same piece products, same k order and same order of additions as the core
+// above: the results are the same bits.
+// The tile reads all of its A rows before it writes any of C: with NH = 2 and N == 128 a product may
+// overwrite its own A operand (C == A), since no other tile touches those rows.
+constexpr int SHORT_K = 128;
+constexpr size_t short_smem_bytes(int nh) { return (size_t)4 * 3 * 2048 * (1 + nh); }
+template <int NH>
+__device__ __forceinline__ void tile_short(const GemmF32& g, int m0, int n0, float* smem_f) {
+  using namespace split;
+  constexpr int PLA = 2048, PLB = 2048 * NH;  // plane: 64 (A) or 64 NH (B) rows x 16 k of bf16
+  constexpr int OPA = 3 * PLA, STG = OPA + 3 * PLB;
+  unsigned char* smem = reinterpret_cast<unsigned char*>(smem_f);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, lr = lane & 31, lk = lane >> 5;
+  const float* __restrict__ A = g.A;
+  const float* __restrict__ B = g.B;
+  const int nsum = g.bsum ? min(g.bsum, (n0 / BN) / g.bsum_c + 1) : 1;
+  // thread -> (row x, four k) of a 64-k half: idx = tid + 256 it, x = idx / 16, k = 4 (idx % 16)
+  floatx4 ra[2][4], rb[2][4 * NH];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int idx = tid + it * 256, x = idx >> 4, k = 64 * h + ((idx & 15) << 2);
+      ra[h][it] = *reinterpret_cast<const floatx4*>(A + (long)(m0 + x) * g.sam + k);
+    }
+#pragma unroll
+    for (int it = 0; it < 4 * NH; ++it) {
+      const int idx = tid + it * 256, x = idx >> 4, k = 64 * h + ((idx & 15) << 2);
+      rb[h][it] = *reinterpret_cast<const floatx4*>(B + (long)(n0 + x) * g.sbn + k);
+    }
+  }
+  constexpr int R = 8 / NH;
+  for (int s0 = 1; s0 < nsum; s0 += R) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      floatx4 t[R][4 * NH];
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const float* Bu = B + (long)min(s0 + u, nsum - 1) * g.bsum_stride;  // past the last: re-read, dropped below
+#pragma unroll
+        for (int it = 0; it < 4 * NH; ++it) {
+          const int idx = tid + it * 256, x = idx >> 4, k = 64 * h + ((idx & 15) << 2);
+          t[u][it] = *reinterpret_cast<const floatx4*>(Bu + (long)(n0 + x) * g.sbn + k);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < R; ++u)
+#pragma unroll
+        for (int it = 0; it < 4 * NH; ++it)
+          if (s0 + u < nsum) rb[h][it] += t[u][it];
+    }
+  }
+  floatx16 acc[NH];
+#pragma unroll
+  for (int j = 0; j < NH; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    if (h) __syncthreads();  // every wavefront has read the first half
+#pragma unroll
+    for (int it = 0; it < 4 * (1 + NH); ++it) {
+      const bool isb = it >= 4;
+      const int idx = tid + (isb ? it - 4 : it) * 256, x = idx >> 4, k4 = (idx & 15) << 2;
+      unsigned char* q = smem + (k4 >> 4) * STG + (isb ? OPA : 0) + ((k4 & 15) >> 3) * (isb ? 1024 * NH : 1024) + x * 16 +
+                         (k4 & 7) * 2;
+      const int plane = isb ? PLB : PLA;
+      const floatx4 v = isb ? rb[h][it - 4] : ra[h][it];
+      const bf16x4v hi = __builtin_convertvector(v, bf16x4v);
+      const floatx4 r1 = v - __builtin_convertvector(hi, floatx4);
+      const bf16x4v mid = __builtin_convertvector(r1, bf16x4v);
+      const floatx4 r2 = r1 - __builtin_convertvector(mid, floatx4);
+      const bf16x4v lo = __builtin_convertvector(r2, bf16x4v);
+      *reinterpret_cast<bf16x4v*>(q) = hi;
+      *reinterpret_cast<bf16x4v*>(q + plane) = mid;
+      *reinterpret_cast<bf16x4v*>(q + 2 * plane) = lo;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const unsigned char* as = smem + s * STG + lk * 1024 + (wm * 32 + lr) * 16;
+      const unsigned char* bs = smem + s * STG + OPA + lk * (1024 * NH) + (wn * 32 * NH + lr) * 16;
+      bf16x8n fa[3], fb[NH][3];
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        fa[p] = *reinterpret_cast<const bf16x8n*>(as + p * PLA);
+#pragma unroll
+        for (int j = 0; j < NH; ++j) fb[j][p] = *reinterpret_cast<const bf16x8n*>(bs + p * PLB + j * 32 * 16);
+      }
+      constexpr int PA[6] = {1, 0, 2, 0, 1, 0}, PB[6] = {1, 2, 0, 1, 0, 0};
+#pragma unroll
+      for (int t = 0; t < 6; ++t)
+#pragma unroll
+        for (int j = 0; j < NH; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[PA[t]], fb[j][PB[t]], acc[j], 0, 0, 0);
+    }
+  }
+  __syncthreads();
+  constexpr int LDC_S = 64 * NH + 4;
+  float* cs = smem_f;
+#pragma unroll
+  for (int j = 0; j < NH; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      cs[(wm * 32 + 8 * (v >> 2) + 4 * lk + (v & 3)) * LDC_S + wn * 32 * NH + j * 32 + lr] = acc[j][v];
+  __syncthreads();
+  const float alpha = g.alpha;
+#pragma unroll
+  for (int it = 0; it < 4 * NH; ++it) {
+    const int idx = tid + it * 256, r = idx / (16 * NH), c = (idx % (16 * NH)) << 2;
+    floatx4 o = *reinterpret_cast<const floatx4*>(cs + r * LDC_S + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = alpha * o[e];
+    *reinterpret_cast<floatx4*>(g.C + (long)(m0 + r) * g.ldc + n0 + c) = o;
   }
 }
 

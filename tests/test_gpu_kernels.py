@@ -183,6 +183,40 @@ def test_factor_from_equals_in_place(dev, C):
     assert lib.mq_factor_upper_inverse_from(H.data_ptr(), C, H.data_ptr(), C, C, 1, info_u.data_ptr(), None) != 0
 
 
+def test_factor_full_width_on_concurrent_streams(dev):
+    """C = 7168 (56 block steps, launches of more workgroups than the chip holds at once), four factorisations
+    in flight on four streams, twice: every result has the same bits, and U H U^T is diagonal.  The in-place
+    panel product must not let one workgroup overwrite rows another still reads: a tiling that did passed every
+    small case and lost a sixth of the codes at this size under load."""
+    C = 7168
+    _say(f"factor C={C} on four streams")
+    gen = torch.Generator(device=dev).manual_seed(91)
+    X = torch.randn(8192, C, generator=gen, device=dev)
+    H = (X.t() @ X) / 8192
+    del X
+    H.diagonal().add_(0.01 * H.diag().mean())
+    lanes = [torch.cuda.Stream(device=dev) for _ in range(4)]
+    outs = []
+    for rep in range(2):
+        for ln in lanes:
+            ln.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(ln):
+                U, info = ops.factor_upper_inverse_from(H)
+                outs.append((U, info))
+    torch.cuda.synchronize()
+    for U, info in outs:
+        assert int(info.item()) == 0
+        assert torch.equal(U, outs[0][0])
+    U = outs[0][0]
+    del outs
+    T = U @ H @ U.t()
+    d = T.diagonal().clone()
+    T.diagonal().zero_()
+    rel = (T.norm() / d.norm()).item()
+    _say(f"  off-diagonal of U H U^T relative to its diagonal: {rel:.2e}")
+    assert rel < 1e-4
+
+
 def test_factor_reports_non_pd(dev):
     C = 256
     H = _spd(C, 77)
