@@ -430,7 +430,7 @@ __device__ __forceinline__ void inv_first_tile(const GemmF32& ginv, int kc, int 
   tile_body<false, true>(gl, tm, 0, 0, buf, 1, 1);
 }
 
-__global__ __launch_bounds__(256) void inv_first_kernel(GemmF32 ginv, int kc) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void inv_first_kernel(GemmF32 ginv, int kc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   inv_first_tile(ginv, kc, blockIdx.x, reinterpret_cast<float*>(smem));
 }
@@ -591,7 +591,8 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
   if (B >= 3) {
     int t2;
     GemmF32 g2 = inv_second(1, t2);
-    if ((rc = mq_launch_gemm_f32(g2, st)) != MQ_OK) return rc;
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t2), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t2);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
   if (B >= 2) {
     int t;
@@ -599,7 +600,8 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     hipLaunchKernelGGL(inv_first_kernel, dim3(t), dim3(256), gemmf32::SMEM_BYTES, st, g1, kc_of(C - NB));
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 g2 = inv_second(0, t);
-    if ((rc = mq_launch_gemm_f32(g2, st)) != MQ_OK) return rc;
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
   hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize, info);
   return mq_check_launch();

@@ -12,7 +12,7 @@ using namespace gemmf32;
 // pair_rows > 0 (triangular-K problems): the workgroup computes row tile tm and then its mirror
 // pair_rows-1-tm, so every workgroup sees the same total K and the triangle no longer unbalances the grid.
 template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int tiles_n, int total, int vecA, int vecB,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f32_kernel(GemmF32 g, int tiles_n, int total, int vecA, int vecB,
                                                       int pair_rows) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   int tm, tn;

@@ -320,27 +320,6 @@ struct Loader {
 #pragma unroll
     for (int it = 0; it < 2; ++it) r[it] = *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
   }
-  // r += the same tile of `n` more arrays, `stride` elements apart; eight arrays' loads are in flight together
-  __device__ __forceinline__ void add_many(const float* __restrict__ p, long stride, int n, long sx, long sk, int x0, int k0,
-                                           int tid) {
-    constexpr int NB8 = 8;
-    for (int s0 = 0; s0 < n; s0 += NB8) {
-      floatx4 t[NB8][2];
-#pragma unroll
-      for (int u = 0; u < NB8; ++u)
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          // (arrays past the last one re-read the last: the value is dropped below)
-          const float* q = addr(p + (long)min(s0 + u, n - 1) * stride, sx, sk, x0, k0, it, tid);
-          t[u][it] = *reinterpret_cast<const floatx4*>(q);
-        }
-#pragma unroll
-      for (int u = 0; u < NB8; ++u)
-#pragma unroll
-        for (int it = 0; it < 2; ++it)
-          if (s0 + u < n) r[it] += t[u][it];
-    }
-  }
   __device__ __forceinline__ void store(unsigned char* op, int tid) const {
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
@@ -406,19 +385,46 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  Loader<A_KC> la;
-  Loader<B_KC> lb;
-  const int nsum = g.bsum ? min(g.bsum, (n0 / BN) / g.bsum_c + 1) : 1;  // arrays summed into the B operand
-#define MQ_SPLIT_FETCH(k0)                                                                     \
-  do {                                                                                         \
-    la.load(A, g.sam, g.sak, m0, (k0), tid);                                                   \
-    lb.load(B, g.sbn, g.sbk, n0, (k0), tid);                                                   \
-    if (nsum > 1) lb.add_many(B + g.bsum_stride, g.bsum_stride, nsum - 1, g.sbn, g.sbk, n0, (k0), tid); \
-  } while (0)
+  // Operand tiles travel memory -> registers -> LDS.  A 16-k step is 768 MFMA cycles per wavefront, a memory
+  // round trip under load several times that: the registers hold the next two steps, so a step's loads have
+  // two steps of products to arrive in.
+  Loader<A_KC> la[2];
+  Loader<B_KC> lb[2];
   const float* Cold = g.Csrc ? g.Csrc + (C - g.C) : C;
   const long ldcold = g.Csrc ? g.ldcs : g.ldc;
   const int nk = (ke - kb) / SBK;
-  if (nk > 0) MQ_SPLIT_FETCH(kb);
+  // Where the next step to fetch lies, kept in registers of their own and moved on by a wave-uniform stride:
+  // address arithmetic in temporaries tempts the register allocator to compute it in the registers a load
+  // still in flight will write, and the hazard costs a wait for every load.  Past the last step the pointers
+  // stay (the last step is fetched again and never used): no branch around a load, at whose join the
+  // compiler would wait for all of them as well.
+  const float* qa[2];
+  const float* qb[2];
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    qa[it] = la[0].addr(A, g.sam, g.sak, m0, kb, it, tid);
+    qb[it] = lb[0].addr(B, g.sbn, g.sbk, n0, kb, it, tid);
+  }
+  const long inca = (long)SBK * g.sak, incb = (long)SBK * g.sbk;
+  int fetched = 0;  // steps fetched so far
+  auto fetch = [&](Loader<A_KC>& xa, Loader<B_KC>& xb) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      xa.r[it] = *reinterpret_cast<const floatx4*>(qa[it]);
+      xb.r[it] = *reinterpret_cast<const floatx4*>(qb[it]);
+    }
+    ++fetched;
+    const long ia = fetched < nk ? inca : 0, ib = fetched < nk ? incb : 0;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      qa[it] += ia;
+      qb[it] += ib;
+    }
+  };
+  if (nk > 0) {
+    fetch(la[0], lb[0]);
+    fetch(la[1], lb[1]);
+  }
   constexpr int LDC_S = BN + 4;
   floatx4 cold4[16];
   if (beta != 0.f) {
@@ -429,13 +435,14 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
     }
   }
   if (nk > 0) {
-    la.store(smem, tid);
-    lb.store(smem + OPB_MAX, tid);
+    la[0].store(smem, tid);
+    lb[0].store(smem + OPB_MAX, tid);
   }
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
+  // step kt: LDS stage kt%2 holds its operands, `nxt` those of step kt+1 (in flight), `fre` is free
+  auto step = [&](int kt, Loader<A_KC>& fa_free, Loader<B_KC>& fb_free, Loader<A_KC>& fa_next, Loader<B_KC>& fb_next) {
     const int cur = kt & 1;
-    if (kt + 1 < nk) MQ_SPLIT_FETCH(kb + (kt + 1) * SBK);
+    fetch(fa_free, fb_free);  // step kt + 2
     const unsigned char* as = smem + cur * STAGEB;
     const unsigned char* bs = as + OPB_MAX;
     bf16x8n fa[2][3], fb[2][3];
@@ -453,13 +460,16 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][PA[t]], fb[j][PB[t]], acc[i][j], 0, 0, 0);
-    if (kt + 1 < nk) {
-      la.store(smem + (cur ^ 1) * STAGEB, tid);
-      lb.store(smem + (cur ^ 1) * STAGEB + OPB_MAX, tid);
-    }
+    // (no branch here either: after the last step this writes a stage nobody reads, and the whole step stays
+    // one block of code in which the conversions can be scheduled between the matrix instructions)
+    fa_next.store(smem + (cur ^ 1) * STAGEB, tid);
+    fb_next.store(smem + (cur ^ 1) * STAGEB + OPB_MAX, tid);
     __syncthreads();
+  };
+  for (int kt = 0; kt < nk; kt += 2) {
+    step(kt, la[0], lb[0], la[1], lb[1]);
+    if (kt + 1 < nk) step(kt + 1, la[1], lb[1], la[0], lb[0]);
   }
-#undef MQ_SPLIT_FETCH
   float* cs = smem_f;  // the loop's last barrier has passed: no wavefront reads operands any more
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -627,7 +637,7 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0 &&  // C moves 16 bytes at a time
                                  (!g.Csrc || ((((uintptr_t)g.Csrc) & 15) == 0 && (g.ldcs & 3) == 0)));
   const bool inside = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N;
-  if (!LDS_OUT && !g.fp32_mfma && inside && ((ke - kb) % split::SBK == 0)) {
+  if (!LDS_OUT && !g.fp32_mfma && !g.bsum && inside && ((ke - kb) % split::SBK == 0)) {
     tile_core_split<A_KC, B_KC>(g, m0, n0, kb, ke, A, B, C, smem);
     return;
   }

@@ -194,7 +194,7 @@ __device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], co
 // use: the kernel is built from branch-free unrolled blocks for that reason (ROWMAP / QZERO are template
 // flags, the rounding mode is a select).
 template <bool FULL, bool ROWMAP, bool QZERO>
-__global__ __launch_bounds__(256) void gptq_block_kernel(LoopArgs a, int i1, int nb, int col_wgs, GemmF32 g, int tiles_n,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gptq_block_kernel(LoopArgs a, int i1, int nb, int col_wgs, GemmF32 g, int tiles_n,
                                                         int vecA, int vecB) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   if ((int)blockIdx.x >= col_wgs) {  // a tile of the previous block's trailing update
