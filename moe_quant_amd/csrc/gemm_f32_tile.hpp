@@ -307,6 +307,28 @@ static_assert(2 * STAGEB <= (int)SMEM_BYTES, "two stages must fit in the fp32 co
 typedef __bf16 bf16x4v __attribute__((ext_vector_type(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+// two floats -> two bf16 (round to nearest even) in one word: one v_cvt_pk_bf16_f32
+__device__ __forceinline__ unsigned pk_bf16(float a, float b) {
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(float2v{a, b}, bf16x2v));
+}
+// v = hi + mid + lo, each a bf16 (four elements: two words per piece).  The rounded pieces are turned back
+// into floats by a shift or a mask of the packed word: 11 instructions per pair of elements.
+__device__ __forceinline__ void split3(const floatx4 v, uint2v& hi, uint2v& mid, uint2v& lo) {
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const unsigned h = pk_bf16(v[2 * p], v[2 * p + 1]);
+    const float r0 = v[2 * p] - __uint_as_float(h << 16), r1 = v[2 * p + 1] - __uint_as_float(h & 0xffff0000u);
+    const unsigned m = pk_bf16(r0, r1);
+    const float s0 = r0 - __uint_as_float(m << 16), s1 = r1 - __uint_as_float(m & 0xffff0000u);
+    hi[p] = h;
+    mid[p] = m;
+    lo[p] = pk_bf16(s0, s1);
+  }
+}
+
 template <bool KC>
 struct Loader {
   floatx4 r[2];
@@ -324,12 +346,8 @@ struct Loader {
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       const int idx = tid + it * 256;
-      const floatx4 v = r[it];
-      const bf16x4v hi = __builtin_convertvector(v, bf16x4v);
-      const floatx4 r1 = v - __builtin_convertvector(hi, floatx4);
-      const bf16x4v mid = __builtin_convertvector(r1, bf16x4v);
-      const floatx4 r2 = r1 - __builtin_convertvector(mid, floatx4);
-      const bf16x4v lo = __builtin_convertvector(r2, bf16x4v);
+      uint2v hi, mid, lo;
+      split3(r[it], hi, mid, lo);
       unsigned char* q;
       int plane;
       if (KC) {
@@ -341,9 +359,9 @@ struct Loader {
         q = op + k * XROW + x4 * 2;
         plane = XPLANE;
       }
-      *reinterpret_cast<bf16x4v*>(q) = hi;
-      *reinterpret_cast<bf16x4v*>(q + plane) = mid;
-      *reinterpret_cast<bf16x4v*>(q + 2 * plane) = lo;
+      *reinterpret_cast<uint2v*>(q) = hi;
+      *reinterpret_cast<uint2v*>(q + plane) = mid;
+      *reinterpret_cast<uint2v*>(q + 2 * plane) = lo;
     }
   }
 };
@@ -566,15 +584,11 @@ __device__ __forceinline__ void tile_short(const GemmF32& g, int m0, int n0, flo
       unsigned char* q = smem + (k4 >> 4) * STG + (isb ? OPA : 0) + ((k4 & 15) >> 3) * (isb ? 1024 * NH : 1024) + x * 16 +
                          (k4 & 7) * 2;
       const int plane = isb ? PLB : PLA;
-      const floatx4 v = isb ? rb[h][it - 4] : ra[h][it];
-      const bf16x4v hi = __builtin_convertvector(v, bf16x4v);
-      const floatx4 r1 = v - __builtin_convertvector(hi, floatx4);
-      const bf16x4v mid = __builtin_convertvector(r1, bf16x4v);
-      const floatx4 r2 = r1 - __builtin_convertvector(mid, floatx4);
-      const bf16x4v lo = __builtin_convertvector(r2, bf16x4v);
-      *reinterpret_cast<bf16x4v*>(q) = hi;
-      *reinterpret_cast<bf16x4v*>(q + plane) = mid;
-      *reinterpret_cast<bf16x4v*>(q + 2 * plane) = lo;
+      uint2v hi, mid, lo;
+      split3(isb ? rb[h][it - 4] : ra[h][it], hi, mid, lo);
+      *reinterpret_cast<uint2v*>(q) = hi;
+      *reinterpret_cast<uint2v*>(q + plane) = mid;
+      *reinterpret_cast<uint2v*>(q + 2 * plane) = lo;
     }
     __syncthreads();
 #pragma unroll
