@@ -36,6 +36,28 @@ def test_gemm_f32_layouts(dev, a_kc, b_kc, M, N, K):
     assert err < 1e-4 * max(1.0, ref.abs().max().item()), err
 
 
+@pytest.mark.parametrize("a_kc,b_kc", [(True, True), (True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("K", [16, 32, 48, 80, 256])
+def test_gemm_f32_interior_tiles_short_and_odd_k(dev, a_kc, b_kc, K):
+    """Interior 128x128 tiles (the bf16-piece core with two k-steps in flight) with 1, 2, 3, 5 and 16 k-steps:
+    the pipeline's start and tail.  Against fp64 the error stays at fp32 rounding level."""
+    M, N = 256, 384
+    _say(f"gemm interior a_kc={a_kc} b_kc={b_kc} K={K}")
+    A = _rand((M, K), 11) * (1.0 + 100.0 * torch.rand(M, 1, generator=torch.Generator().manual_seed(12)))
+    B = _rand((K, N), 13)
+    C0 = _rand((M, N), 14)
+    Ad = (A if a_kc else A.t().contiguous()).to(dev)
+    Bd = (B.t().contiguous() if b_kc else B).to(dev)
+    Cd = C0.clone().to(dev)
+    sam, sak = (K, 1) if a_kc else (1, M)
+    sbk, sbn = (1, K) if b_kc else (N, 1)
+    ops.gemm_f32_(Ad, sam, sak, Bd, sbk, sbn, Cd, M, N, K, alpha=-1.0, beta=1.0)
+    ref = C0.double() - A.double() @ B.double()
+    mag = C0.double().abs() + A.double().abs() @ B.double().abs()
+    rel = ((Cd.cpu().double() - ref).abs() / mag).max().item()
+    assert rel < 4e-7, rel
+
+
 def test_gemm_f32_tri_and_ktrim(dev):
     n = 384
     A = _rand((n, 128), 4)
@@ -166,7 +188,8 @@ def test_factor_vs_torch_chain(dev, C):
 def test_factor_from_equals_in_place(dev, C):
     """The entry point that leaves H untouched builds the same bits as the in-place one, on a destination full of NaN."""
     _say(f"factor_from C={C}")
-    H = _spd(C, seed=17).to(dev)
+    H = torch.empty(C, C + 64, device=dev)[:, :C]  # a row pitch of its own
+    H.copy_(_spd(C, seed=17))
     H0 = H.clone()
     A = H.clone()
     info_a = ops.factor_upper_inverse_(A)
