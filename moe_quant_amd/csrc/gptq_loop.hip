@@ -441,16 +441,32 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   for (int i1 = 0; i1 < a.C; i1 += block, ++blk) {
     const int i2 = (i1 + block < a.C) ? i1 + block : a.C;
     const int nb = i2 - i1;
-    la.E = a.E + (long)(blk & 1) * B * a.R;
-    la.Eprev = blk ? a.E + (long)((blk + 1) & 1) * B * a.R : nullptr;
+    // four error blocks in a ring: this block's, the previous one (the column workgroups fold it into their own
+    // columns) and the pair before, which a trailing update may still be reading
+    la.E = a.E + (long)(blk & 3) * B * a.R;
+    la.Eprev = blk ? a.E + (long)((blk - 1) & 3) * B * a.R : nullptr;
     la.nbprev = nbprev;
-    // the previous block's update of everything beyond this block: Wt[i2+m, r] += sum_j U[i1-nbprev+j, i2+m] * Eprev[j, r]
-    GemmF32 g{a.U + (long)(i1 - nbprev) * a.ldu + i2, la.Eprev, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw,
-              a.C - i2, a.R, nbprev, 1.f, 1.f, 0, 0, 1, 0, 0, 0};
+    // Trailing updates, Wt[i2+m, r] += sum_j U[j0+j, i2+m] * E[j, r], run beside the column walk of this block.
+    // With 128-column blocks they go two blocks at a time: a rank-128 update of everything beyond is bound by
+    // reading and writing those columns, a rank-256 one moves them half as often.  A block must hold every update
+    // but the previous block's when its walk starts, so: odd blocks apply the previous block's errors to the next
+    // block only; even blocks apply the two previous blocks' errors (neighbours in the ring) to everything beyond.
+    // Other block widths: the previous block's errors to everything beyond, every time.
+    GemmF32 g{a.U, la.Eprev, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw, a.C - i2, a.R, nbprev, 1.f, 1.f,
+              0, 0, 1, 0, 0, 0};
     int tiles = 0, tiles_n = 1, vecA = 0, vecB = 0;
     if (blk && i2 < a.C) {
+      long j0 = i1 - nbprev;
+      if (block == B && (blk & 1)) {
+        g.M = (a.C - i2 < block) ? a.C - i2 : block;
+      } else if (block == B) {
+        j0 = i1 - 2 * B;
+        g.B = a.E + (long)((blk - 2) & 3) * B * a.R;
+        g.K = 2 * B;
+      }
+      g.A = a.U + j0 * a.ldu + i2;
       tiles_n = (a.R + gemmf32::BN - 1) / gemmf32::BN;
-      tiles = ((a.C - i2 + gemmf32::BM - 1) / gemmf32::BM) * tiles_n;
+      tiles = ((g.M + gemmf32::BM - 1) / gemmf32::BM) * tiles_n;
       vecA = mq_gemm_operand_aligned(g.A, g.sak, 0);
       vecB = mq_gemm_operand_aligned(g.B, g.sbk, 0);
     }
