@@ -442,11 +442,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void i
 //                          triangular) times K chunk s of 512; chunk s lands 128*s columns to the right of chunk
 //                          0, in the mirror area of block column b+s, free since that row's inverse is complete;
 //                          the second product sums the chunks while loading them;
-//   the rest             : the other T-1 upper tiles of the trailing update  A[0:i1,0:i1] -= P P^T.
+//   the rest             : the other upper tiles of the trailing update  A[0:i1,0:i1] -= P P^T  -- all of
+//                          them, or (column_only) just the block column the next panel needs; see factor_impl.
 // The diagonal-block work is thereby hidden behind the bulk of the trailing update, and the inverse behind both.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void trail_diag_kernel(GemmF32 g, int total, GemmF32 ginv,
                                                                                                   int inv_tiles, int kc, float* A,
-                                                                                                  long ld, int i1, int* info) {
+                                                                                                  long ld, int i1, int* info,
+                                                                                                  int column_only) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* buf = reinterpret_cast<float*>(smem);
   using namespace gemmf32;
@@ -471,7 +473,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
     inv_first_tile(ginv, kc, bid - 1, buf);
   } else {
     int tm, tn;
-    tri_decode(xcd_remap(bid - 1 - inv_tiles, total - 1), tm, tn);
+    const int idx = bid - 1 - inv_tiles, T = i1 / NB;
+    if (column_only) {  // block column T-1 above its diagonal tile, then the diagonal tile after that one
+      tm = idx < T - 1 ? idx : T - 2;
+      tn = idx < T - 1 ? T - 1 : T - 2;
+    } else {
+      tri_decode(xcd_remap(idx, total - 1), tm, tn);
+    }
     tile_body<true, true>(g, tm, tn, 0, buf, 1, 1);
   }
 }
@@ -573,18 +581,27 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     hipLaunchKernelGGL(panel_inv_kernel, dim3(2 * b + 4 * t2), dim3(256), gemmf32::short_smem_bytes(2), st, panel, 2 * b,
                        g2, 4 * t2);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
-    GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
+    // The trailing update A[0:i1,0:i1] -= P P^T with one 128-wide panel is bound by reading and writing the
+    // trailing matrix, so after the first step (which also carries the matrix from S to A) the panels go in
+    // two at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0 owns its
+    // diagonal tile.  Odd steps: this panel into block column b-1 alone, and already into the diagonal tile
+    // after the next one, (b-2, b-2).  Even steps: this panel and the previous one -- neighbours in memory,
+    // A[:, i1 : i1+256], one K = 256 product -- into every tile but (b-1, b-1), which had the previous panel
+    // one step early and takes this one from workgroup 0 as always.
+    const int step = B - 1 - b;
+    const int column_only = step >= 1 && (step & 1);
+    GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, (step >= 2 && !column_only) ? 2 * NB : NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     if (first) {
       trail.Csrc = S;
       trail.ldcs = lds;
     }
     const int tiles = i1 / NB, total = tiles * (tiles + 1) / 2;
+    const int others = column_only ? (b - 1) + (b >= 2 ? 1 : 0) : total - 1;  // tiles besides workgroup 0's
     int t1 = 0;
     GemmF32 g1 = trail;
     if (b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
-    hipLaunchKernelGGL(trail_diag_kernel, dim3(total + t1), dim3(256), FUSED_SMEM, st, trail, total, g1, t1,
-                       kc_of(C - i1 - NB), A, ld,
-                       i1, info);
+    hipLaunchKernelGGL(trail_diag_kernel, dim3(1 + t1 + others), dim3(256), FUSED_SMEM, st, trail, total, g1, t1,
+                       kc_of(C - i1 - NB), A, ld, i1, info, column_only);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
   // what is left of the inverse once the elimination has reached the top: second product of row 1, both of row 0
