@@ -143,8 +143,8 @@ int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int*
  *   qzero : nullable, same indexing; NULL means the constant qzero_const.
  *   round_dtype : rounding of the dequantized value ((q - z) * s), the `dtype` of tl_dequantize.
  *   block : columns per lazy-batch block; values <= 0 or > 128 use 128 (only reassociates fp32 sums).
- *   Qt    : C x R u8 out, integer codes.   E : 4 x 128 x R fp32 scratch (a ring of error blocks: a block's
- *           sequential walk overlaps the trailing update of the two blocks before it).
+ *   Qt    : C x R u8 out, integer codes.   E : 8 x 128 x R fp32 scratch (a ring of error blocks: a block's
+ *           sequential walk overlaps the trailing update of a batch of up to four blocks before it).
  */
 int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale, long ld_scale,
                  const int* scale_row, const float* qzero, float qzero_const, float maxq, int round_dtype, int block,

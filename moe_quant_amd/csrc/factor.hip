@@ -29,6 +29,7 @@ constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
 constexpr int LDM = 132;   // LDS row pitch: rows 16-byte aligned, consecutive rows 4 banks apart (8 rows span the 32 banks)
 constexpr int SOFF = 4;    // column shift of the S triangle inside a row (keeps both triangles 16-byte aligned)
+static int TRAIL_PANELS = 4;  // panels per trailing update of the whole matrix (env MQ_PANELS)
 static int INV_KC = 4;  // the first inverse product is cut into K chunks of 4 blocks (512), one workgroup each
 
 // ---------------------------------------------------------------------------------------------
@@ -535,6 +536,7 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
   static bool attr_done = false;
   if (!attr_done) {
     if (const char* e = getenv("MQ_INV_KC")) INV_KC = atoi(e) > 0 ? atoi(e) : INV_KC;
+    if (const char* e = getenv("MQ_PANELS")) TRAIL_PANELS = atoi(e) > 0 ? atoi(e) : TRAIL_PANELS;
     (void)hipFuncSetAttribute((const void*)revchol_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)DIAG_SMEM);
     (void)hipFuncSetAttribute((const void*)trail_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -583,14 +585,18 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     // The trailing update A[0:i1,0:i1] -= P P^T with one 128-wide panel is bound by reading and writing the
     // trailing matrix, so after the first step (which also carries the matrix from S to A) the panels go in
-    // two at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0 owns its
-    // diagonal tile.  Odd steps: this panel into block column b-1 alone, and already into the diagonal tile
-    // after the next one, (b-2, b-2).  Even steps: this panel and the previous one -- neighbours in memory,
-    // A[:, i1 : i1+256], one K = 256 product -- into every tile but (b-1, b-1), which had the previous panel
-    // one step early and takes this one from workgroup 0 as always.
+    // TRAIL_PANELS at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0
+    // owns its diagonal tile.  Steps in between (column_only): the j panels block column b-1 still lacks --
+    // this one and the j-1 before it, neighbours in memory, A[:, i1 : i1+128j], one product with K = 128j --
+    // into that block column alone, and already into the diagonal tile after the next one, (b-2, b-2).  Every
+    // TRAIL_PANELS-th step: the last TRAIL_PANELS panels into every tile but (b-1, b-1), which had all but
+    // this panel one step early and takes this one from workgroup 0 as always.
+    // (2, 3, 4, 6 panels: 306, 311, 314, 315 linears/s at four streams against 286 with one; a single
+    // factorisation takes 3.21 -> 3.28 ms with four, the steps in between leave the chip idle.)
     const int step = B - 1 - b;
-    const int column_only = step >= 1 && (step & 1);
-    GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, (step >= 2 && !column_only) ? 2 * NB : NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
+    const int j = step >= 1 ? (step - 1) % TRAIL_PANELS + 1 : 1;  // panels owed to block column b-1 (step 0: the plain update)
+    const int column_only = step >= 1 && j < TRAIL_PANELS;
+    GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, j * NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     if (first) {
       trail.Csrc = S;
       trail.ldcs = lds;

@@ -23,6 +23,9 @@
 namespace {
 
 constexpr int B = 128;
+constexpr int LOOP_BATCH_MAX = 4;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
+static int LOOP_BATCH = 2;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..4;
+                                    // 1, 2, 3, 4: 300, 312, 312, 309 linears/s at four streams)
 
 __device__ __forceinline__ float round_dtype(float x, int rd) {
   // branch-free so that the unrolled column steps stay one basic block
@@ -434,6 +437,10 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
     (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
+    if (const char* e = getenv("MQ_LOOP_BATCH")) {
+      const int v = atoi(e);
+      if (v >= 1 && v <= LOOP_BATCH_MAX) LOOP_BATCH = v;
+    }
     attr_done = true;
   }
   LoopArgs la = a;
@@ -441,28 +448,31 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   for (int i1 = 0; i1 < a.C; i1 += block, ++blk) {
     const int i2 = (i1 + block < a.C) ? i1 + block : a.C;
     const int nb = i2 - i1;
-    // four error blocks in a ring: this block's, the previous one (the column workgroups fold it into their own
-    // columns) and the pair before, which a trailing update may still be reading
-    la.E = a.E + (long)(blk & 3) * B * a.R;
-    la.Eprev = blk ? a.E + (long)((blk - 1) & 3) * B * a.R : nullptr;
+    // Error blocks live in a ring of 2 * LOOP_BATCH: this block's, the previous one (the column workgroups fold it
+    // into their own columns) and the batches a trailing update may still be reading.
+    const int RING = 2 * LOOP_BATCH;  // a multiple of the batch: an aligned batch never wraps
+    la.E = a.E + (long)(blk % RING) * B * a.R;
+    la.Eprev = blk ? a.E + (long)((blk - 1) % RING) * B * a.R : nullptr;
     la.nbprev = nbprev;
     // Trailing updates, Wt[i2+m, r] += sum_j U[j0+j, i2+m] * E[j, r], run beside the column walk of this block.
-    // With 128-column blocks they go two blocks at a time: a rank-128 update of everything beyond is bound by
-    // reading and writing those columns, a rank-256 one moves them half as often.  A block must hold every update
-    // but the previous block's when its walk starts, so: odd blocks apply the previous block's errors to the next
-    // block only; even blocks apply the two previous blocks' errors (neighbours in the ring) to everything beyond.
-    // Other block widths: the previous block's errors to everything beyond, every time.
+    // A rank-128 update of everything beyond is bound by reading and writing those columns, so with 128-column
+    // blocks the errors go in batches of D blocks (aligned: blocks [mD, mD+D), neighbours in the ring).  A block
+    // must hold every update but the previous block's when its walk starts.  Hence, with r = blk % D: r == 0 and
+    // blk >= D: the batch just completed into everything beyond (K = 128 D); otherwise the r errors of the batch
+    // under way into the next block only (K = 128 r).
+    // Other block widths: the previous block's errors into everything beyond, every time.
     GemmF32 g{a.U, la.Eprev, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw, a.C - i2, a.R, nbprev, 1.f, 1.f,
               0, 0, 1, 0, 0, 0};
     int tiles = 0, tiles_n = 1, vecA = 0, vecB = 0;
     if (blk && i2 < a.C) {
       long j0 = i1 - nbprev;
-      if (block == B && (blk & 1)) {
-        g.M = (a.C - i2 < block) ? a.C - i2 : block;
-      } else if (block == B) {
-        j0 = i1 - 2 * B;
-        g.B = a.E + (long)((blk - 2) & 3) * B * a.R;
-        g.K = 2 * B;
+      if (block == B) {
+        const int D = LOOP_BATCH, r = blk % D;
+        const int first = r ? blk - r : blk - D;  // first block of the errors applied now
+        if (r) g.M = (a.C - i2 < block) ? a.C - i2 : block;
+        j0 = (long)first * B;
+        g.B = a.E + (long)(first % RING) * B * a.R;
+        g.K = (blk - first) * B;
       }
       g.A = a.U + j0 * a.ldu + i2;
       tiles_n = (a.R + gemmf32::BN - 1) / gemmf32::BN;

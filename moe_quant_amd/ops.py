@@ -256,7 +256,7 @@ def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor]
     if scale_row is None and scale.shape[0] != C:
         raise ValueError("scale must be (C,R) when no scale_row map is given")
     Qt = torch.empty(C, R, dtype=torch.uint8, device=Wt.device)
-    E = _ws.get(Wt.device, 4 * 128 * R * 4, "loop")
+    E = _ws.get(Wt.device, 8 * 128 * R * 4, "loop")
     rc = lib.mq_gptq_loop(Wt.data_ptr(), Wt.stride(0), C, R, U.data_ptr(), U.stride(0), scale.data_ptr(),
                           scale.stride(0), _p(scale_row), _p(qzero), qzero_const, maxq, _dt(round_dtype), block,
                           Qt.data_ptr(), E.data_ptr(), _stream(Wt))
