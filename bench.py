@@ -242,7 +242,7 @@ def main():
     # (2/3) C^3 flop / measured device time of the chain
     # HBM bytes per factorisation of a 7168^2 matrix, from the two rocprofv3 --pmc runs summarised in
     # profiles/config1_bench_hbm_traffic.md (2.00*FETCH_SIZE + 1.00*WRITE_SIZE, calibrated on copy/fill kernels)
-    traffic = 9.68e9 if C == 7168 else None
+    traffic = 7.34e9 if C == 7168 else None
     roofline = {
         "kernel": "mq_factor_upper_inverse = trail_diag_kernel + panel_inv_kernel + inv_first_kernel + revchol_diag_kernel + "
                   "unit_diag_kernel (one launch sequence per call; largest share of the step). fp32 in, fp32 out; the "
