@@ -26,8 +26,8 @@ PEAK_HBM = 8000.0  # GB/s
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=16)
-    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--streams", type=int, default=4,
                     help="independent linears are queued round-robin on this many HIP streams (1 = one at a time)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
