@@ -9,8 +9,10 @@
 //
 //   per 128-block b (last to first):
 //     diag kernel  : R_bb = revchol(H_bb), then R_bb^-1 written in place (one workgroup, LDS resident)
-//     panel GEMM   : R_ab = H_ab * (R_bb^-1)^T            for a < b   (fp32 MFMA)
-//     trailing GEMM: H_aa' -= R_ab R_a'b^T                for a <= a' < b  (fp32 MFMA, upper tiles only)
+//     panel GEMM   : R_ab = H_ab * (R_bb^-1)^T            for a < b
+//     trailing GEMM: H_aa' -= R_ab R_a'b^T                for a <= a' < b  (upper tiles only; applied lazily:
+//                    at once only to the block column the next panel needs, to the rest several panels at a
+//                    time, see factor_impl)
 //   triangular inverse, one block row at a time, bottom to top, riding along in the same launches:
 //     row b:  T^T = U22^T R12^T   (U22 = finished inverse of everything below/right of b, R12 = R[b, b+1:];
 //                                  written to the unused mirror position below the diagonal)

@@ -9,10 +9,11 @@
 //                         block's errors (a 128x64x128 product on the matrix cores), then walk the columns in
 //                         order (quantize -> dequantize -> error -> fused-multiply-add of the error into the
 //                         remaining block columns) and leave codes, dequantized weights and the error block.
-//     trailing tiles    : Wt[i2:, :] += U[prev block, i2:]^T * E_prev, the previous block's lazy-batch update
-//                         of everything beyond block b, as 128x128 fp32 MFMA tiles (gemm_f32_tile.hpp).
-//   The sequential walk of block b thus overlaps the bulk of block b-1's trailing update; the error block is
-//   double-buffered.
+//     trailing tiles    : Wt[i2:, :] += U[earlier blocks, i2:]^T * E, the lazy-batch update of the columns beyond
+//                         block b with the errors of earlier blocks, as 128x128 tiles (gemm_f32_tile.hpp): the
+//                         next block always, everything beyond once per batch of blocks (see run_loop).
+//   The sequential walk of block b thus overlaps the bulk of the trailing updates; the error blocks live in a
+//   ring.
 //
 // Arithmetic per column is the reference's: q = clamp(floor(x/s + z + 0.5), 0, maxq) with IEEE division,
 // y = round_to(dtype)((q - z) * s), e = y - x, w_k = fma(U[j,k], e, w_k).
