@@ -58,6 +58,26 @@ def test_gemm_f32_interior_tiles_short_and_odd_k(dev, a_kc, b_kc, K):
     assert rel < 4e-7, rel
 
 
+def test_gemm_f32_interior_tiles_wide_dynamic_range(dev):
+    """Magnitudes from 1e-12 to 1e12 inside one row: every piece product is exact, but a matrix instruction
+    aligns its 16 addends to the largest before adding, so the error is a few ulp of the largest terms rather
+    than of each term.  It stays within 2e-6 of sum |a||b| (K = 512; the worst-case bound of any fp32 summation
+    is K * 6e-8 = 3e-5) and is compared with torch's fp32 product of the same operands."""
+    M, N, K = 256, 256, 512
+    g = torch.Generator().manual_seed(21)
+    A = torch.randn(M, K, generator=g) * torch.pow(10.0, torch.rand(M, K, generator=g) * 24 - 12)
+    B = torch.randn(K, N, generator=g) * torch.pow(10.0, torch.rand(K, N, generator=g) * 24 - 12)
+    Cd = torch.zeros(M, N, device=dev)
+    ops.gemm_f32_(A.to(dev), K, 1, B.t().contiguous().to(dev), 1, K, Cd, M, N, K, alpha=1.0, beta=0.0)
+    ref = A.double() @ B.double()
+    mag = A.double().abs() @ B.double().abs()
+    rel = ((Cd.cpu().double() - ref).abs() / mag).max().item()
+    Ct = A.to(dev) @ B.to(dev)
+    rel_t = ((Ct.cpu().double() - ref).abs() / mag).max().item()
+    _say(f"gemm wide dynamic range: max error / sum|a||b| = {rel:.2e} (torch fp32: {rel_t:.2e})")
+    assert rel < 2e-6, rel
+
+
 def test_gemm_f32_tri_and_ktrim(dev):
     n = 384
     A = _rand((n, 128), 4)
