@@ -202,8 +202,8 @@ def main():
         A.copy_(Hd)
         ops.factor_upper_inverse_(A, info)
 
-    t_copy = timed(lambda: A.copy_(Hd))
-    t_factor = timed(factor) - t_copy
+    t_copy = timed(lambda: A.copy_(Hd), reps=8)
+    t_factor = timed(factor, reps=8) - t_copy
     Wd = layer.weight.data
     s_rg, s_gr = ops.quant_grid_sym(Wd, 128, 4, torch.bfloat16)
     scale_row = torch.arange(C, device=dev, dtype=torch.int32) // 128
@@ -215,6 +215,33 @@ def main():
     t_pack = timed(lambda: ops.pack_from_qt(Qt), reps=10)
     codes = ops.untranspose_codes(Qt)
     t_pack_rc = timed(lambda: ops.pack_int4(codes), reps=10)
+
+    # the three big phases once more, `streams` independent calls in flight: device time per call when the chip is
+    # kept full (their sum is what a whole step costs at that many streams)
+    def per_call_in_flight(make_fn, reps=6):
+        fns = [make_fn(i) for i in range(len(lanes))]
+        for f in fns:
+            f()
+        torch.cuda.synchronize()
+        for ln in lanes:
+            if ln is not main_stream:
+                ln.wait_stream(main_stream)
+        t_begin = time.perf_counter()
+        for _ in range(reps):
+            for ln, f in zip(lanes, fns):
+                with torch.cuda.stream(ln):
+                    f()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t_begin) * 1e3 / (reps * len(lanes))
+
+    Hs = [torch.zeros(C, C, device=dev) for _ in lanes]
+    Wts = [torch.empty_like(Wt0) for _ in lanes]
+    infos = [torch.zeros(1, dtype=torch.int32, device=dev) for _ in lanes]
+    t_syrk_fl = per_call_in_flight(lambda i: (lambda: ops.hessian_syrk_(Hs[i], X, 0.0, 2.0 / n, mirror=False)))
+    t_factor_fl = per_call_in_flight(lambda i: (lambda: ops.factor_upper_inverse_from(Hd, infos[i])))
+    t_loop_fl = per_call_in_flight(lambda i: (lambda: (Wts[i].copy_(Wt0), ops.gptq_loop_(
+        Wts[i], A, s_gr, scale_row, None, 8.0, 15.0, torch.bfloat16, 128)))) - t_wcopy
+    del Hs, Wts
 
     pts = torch.linspace(1, 0.2, 100, dtype=torch.float32, device=dev)
     s_try = s_rg.clone()
@@ -231,6 +258,10 @@ def main():
         "pack_from_loop_codes_ms": round(t_pack, 4),
         "pack_int4_ms": round(t_pack_rc, 4),
         "mse_scale_search_ms_not_in_step": round(t_mse, 4),
+        "streams_in_flight": len(lanes),
+        "hessian_syrk_ms_in_flight": round(t_syrk_fl, 4),
+        "factor_ms_in_flight": round(t_factor_fl, 4),
+        "gptq_loop_ms_in_flight": round(t_loop_fl, 4),
         "hessian_syrk_tflops": round(flop_syrk / t_syrk / 1e9, 2),
         "hessian_syrk_frac_bf16_peak": round(flop_syrk / t_syrk / 1e9 / PEAK_BF16_MFMA, 4),
         "factor_tflops": round(flop_factor / t_factor / 1e9, 2),
