@@ -181,7 +181,7 @@ def _spd(C, seed, n=None):
     return H
 
 
-@pytest.mark.parametrize("C", [128, 256, 384, 896, 1024, 2432])
+@pytest.mark.parametrize("C", [128, 256, 384, 640, 896, 1024, 1536, 2176, 2432])  # 1 .. 19 blocks: every phase of the panel batches
 def test_factor_vs_torch_chain(dev, C):
     _say(f"factor C={C}")
     H = _spd(C, C)
