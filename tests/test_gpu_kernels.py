@@ -431,7 +431,8 @@ def _loop_case(R, C, seed, g=128, act_order=False):
 
 
 @pytest.mark.parametrize(
-    "R,C,block,g", [(256, 512, 128, 128), (100, 384, 128, 128), (64, 300, 128, 100), (130, 256, 64, 128), (64, 128, 128, 128)]
+    "R,C,block,g", [(256, 512, 128, 128), (100, 384, 128, 128), (64, 300, 128, 100), (130, 256, 64, 128), (64, 128, 128, 128),
+                    (64, 1024, 128, 128), (96, 900, 128, 100), (70, 1300, 128, 100)]  # 8+ blocks: the error ring wraps
 )
 def test_loop_vs_oracle_same_U(dev, R, C, block, g):
     _say(f"loop R={R} C={C} block={block} g={g}")
