@@ -1,12 +1,17 @@
-"""Drop-in for the model-independent parts of MoE-Quant's pack_quantized_model.py: pack_weight (the
-compressed_tensors "pack-quantized" int32 layout, packed by the HIP kernel), the quantization_config it writes,
-and the per-block step that swaps quantized linears into a block's state dict and saves one safetensors shard.
-Loading the 163-shard DeepSeek checkpoint, the HF config/tokenizer copies and the FP8 dequantization of the
-untouched tensors stay with the caller."""
+"""Drop-in for MoE-Quant's pack_quantized_model.py: pack_weight (the compressed_tensors "pack-quantized" int32
+layout, packed by the HIP kernel), the quantization_config it writes, the per-block step that swaps quantized
+linears into a block's state dict and saves one safetensors shard, and the command line that walks a whole
+checkpoint (`python -m moe_quant_amd.pack_quantized_model --model_name_or_path ... --quantized_model_path ...
+--packed_model_path ...`, the reference's arguments).  The command line reads the checkpoint's own
+`model.safetensors.index.json` instead of the reference's hard-coded 163 DeepSeek shards and edits `config.json`
+as JSON instead of going through transformers' remote-code config class; the files it writes are the same."""
 from __future__ import annotations
 
+import argparse
 import json
 import os
+import re
+import shutil
 from collections import defaultdict
 from typing import Any, Dict, Iterable, Optional
 
@@ -124,3 +129,112 @@ def save_safetensors_index(packed_model_path: str, safetensors_index: Dict[str, 
     """pack_quantized_model.py:232-233."""
     with open(os.path.join(packed_model_path, "model.safetensors.index.json"), "w") as f:
         json.dump({"metadata": {}, "weight_map": safetensors_index}, f)
+
+
+# ---- the whole checkpoint (pack_quantized_model.py:112-243) -------------------------------------------------
+class _Shards:
+    """Tensors of a sharded safetensors checkpoint by name; shard files are opened on demand."""
+
+    def __init__(self, weight_dir: str):
+        self.dir = weight_dir
+        idx = os.path.join(weight_dir, "model.safetensors.index.json")
+        if os.path.exists(idx):
+            with open(idx) as f:
+                self.weight_map = dict(json.load(f)["weight_map"])
+        else:  # a single file
+            from safetensors import safe_open
+
+            with safe_open(os.path.join(weight_dir, "model.safetensors"), framework="pt", device="cpu") as f:
+                self.weight_map = {k: "model.safetensors" for k in f.keys()}
+
+    def load(self, keys: Iterable[str]) -> Dict[str, torch.Tensor]:
+        from safetensors import safe_open
+
+        by_file = defaultdict(list)
+        for k in keys:
+            by_file[self.weight_map[k]].append(k)
+        out = {}
+        for fn, ks in by_file.items():
+            with safe_open(os.path.join(self.dir, fn), framework="pt", device="cpu") as f:
+                for k in ks:
+                    out[k] = f.get_tensor(k)
+        return out
+
+
+def pack_checkpoint(model_name_or_path: str, quantized_model_path: str, packed_model_path: str,
+                    dtype: torch.dtype = torch.float16) -> Dict[str, str]:
+    """pack_quantized_model.py:112-243 for any checkpoint with `model.layers.<i>.` blocks: shard 1 holds the
+    embeddings, one shard per block follows (FP8 tensors dequantized to `dtype`, quantized linears replaced by
+    weight_packed / weight_shape / weight_scale), the last shard holds what is left (lm_head, final norm).
+    Writes the weight map, `config.json` with the compressed-tensors `quantization_config`, and copies tokenizer,
+    generation config and modeling scripts when the source directory has them.  Returns the weight map."""
+    from . import quant_utils
+
+    meta = torch.load(os.path.join(quantized_model_path, "metadata.pt"), weights_only=True)
+    bits, group_size, only_experts = int(meta["bits"]), int(meta["group_size"]), bool(meta["quantize_only_experts"])
+    sym = True  # asymmetric quantization is not supported (pack_quantized_model.py:137-138)
+    shards = _Shards(model_name_or_path)
+    block_keys = defaultdict(list)
+    rest = []
+    for k in shards.weight_map:
+        m = re.match(r"model\.layers\.(\d+)\.", k)
+        (block_keys[int(m.group(1))] if m else rest).append(k)
+    n_blocks = max(block_keys) + 1 if block_keys else 0
+    num_output_shards = n_blocks + 2
+    quantized = quantized_layers_by_block(quantized_model_path)
+    index: Dict[str, str] = {}
+    os.makedirs(packed_model_path, exist_ok=True)
+    first = [k for k in rest if k == "model.embed_tokens.weight"]
+    save_packed_shard(shards.load(first), packed_model_path, 1, num_output_shards, index)
+    def dequantized(sd):  # FP8 weights visit the GPU: one fused pass there instead of the padded torch path
+        for k, v in list(sd.items()):
+            if v.dtype == torch.float8_e4m3fn and torch.cuda.is_available():
+                sd[k] = v.cuda()
+        quant_utils.dequantize_state_dict(sd, dtype)
+        return {k: v.cpu() for k, v in sd.items()}
+
+    for b in range(n_blocks):
+        sd = dequantized(shards.load(block_keys[b]))
+        sd = pack_block_state_dict(sd, quantized_model_path, quantized.get(b, []), bits, sym, group_size)
+        save_packed_shard(sd, packed_model_path, b + 2, num_output_shards, index)
+        del sd
+    last = [k for k in rest if k not in first]
+    save_packed_shard(dequantized(shards.load(last)), packed_model_path, num_output_shards, num_output_shards, index)
+    save_safetensors_index(packed_model_path, index)
+    cfg_path = os.path.join(model_name_or_path, "config.json")
+    cfg = {}
+    if os.path.exists(cfg_path):
+        with open(cfg_path) as f:
+            cfg = json.load(f)
+    cfg.pop("quantization_config", None)  # the source's FP8 description no longer applies (pack_quantized_model.py:118-119)
+    cfg["quantization_config"] = prepare_quantization_config(bits, group_size, only_experts)
+    with open(os.path.join(packed_model_path, "config.json"), "w") as f:
+        json.dump(cfg, f, indent=2)
+    for fn in sorted(os.listdir(model_name_or_path)):
+        if fn == "config.json" or fn.endswith(".safetensors") or fn == "model.safetensors.index.json":
+            continue
+        if fn.endswith((".py", ".model", ".txt")) or fn.startswith(("tokenizer", "special_tokens", "generation_config", "vocab",
+                                                                     "merges", "added_tokens")):
+            src = os.path.join(model_name_or_path, fn)
+            if os.path.isfile(src):
+                shutil.copy(src, packed_model_path)
+    return index
+
+
+def parse_args(argv=None) -> argparse.Namespace:
+    """pack_quantized_model.py:18-49."""
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--model_name_or_path", type=str, required=True, help="Path to the original checkpoint directory")
+    parser.add_argument("--quantized_model_path", type=str, required=True, help="Path to quantized model.")
+    parser.add_argument("--packed_model_path", type=str, required=True, help="Where to save the packed model.")
+    parser.add_argument("--dtype", default="float16", type=str, choices=["float16", "bfloat16"], help="Torch dtype used.")
+    return parser.parse_args(argv)
+
+
+def main(argv=None) -> None:
+    args = parse_args(argv)
+    pack_checkpoint(args.model_name_or_path, args.quantized_model_path, args.packed_model_path, getattr(torch, args.dtype))
+
+
+if __name__ == "__main__":
+    main()

@@ -159,3 +159,81 @@ def test_pack_block_after_driver(dev, tmp_path):
     w = cfg["config_groups"]["group_0"]["weights"]
     assert cfg["format"] == "pack-quantized" and w["num_bits"] == 4 and w["group_size"] == 128 and w["symmetric"]
     assert "re:.*shared_experts.*" in cfg["ignore"] and cfg["ignore"][0] == "lm_head"
+
+
+def test_pack_command_line_on_a_synthetic_checkpoint(dev, tmp_path):
+    """The whole pack step through its command line: a two-block sharded checkpoint (one FP8 tensor with its block
+    scales, a stale quantization_config, a tokenizer file) + a quantized directory -> packed shards, weight map and
+    config.json; everything read back and checked against the inputs."""
+    import json
+
+    from safetensors.torch import load_file, save_file
+
+    from moe_quant_amd import pack_quantized_model as P
+
+    g = torch.Generator().manual_seed(5)
+    src, qdir, pdir = tmp_path / "src", tmp_path / "q", tmp_path / "packed"
+    src.mkdir()
+    R, C = 256, 384
+    tensors = {"model.embed_tokens.weight": torch.randn(50, 64, generator=g).bfloat16(),
+               "lm_head.weight": torch.randn(50, 64, generator=g).bfloat16(),
+               "model.norm.weight": torch.ones(64).bfloat16()}
+    qnames = []
+    for b in range(2):
+        pre = f"model.layers.{b}."
+        tensors[pre + "input_layernorm.weight"] = torch.ones(64).bfloat16()
+        for proj in ("gate_proj", "down_proj"):
+            name = f"{pre}mlp.experts.0.{proj}"
+            tensors[name + ".weight"] = (torch.randn(R, C, generator=g) * 0.02).bfloat16()
+            qnames.append(name)
+    fp8_name = "model.layers.1.self_attn.o_proj"
+    w8 = (torch.randn(R, C, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    s8 = torch.rand(R // 128, C // 128, generator=g) * 0.1 + 0.01
+    tensors[fp8_name + ".weight"] = w8
+    tensors[fp8_name + ".weight_scale_inv"] = s8
+    keys = sorted(tensors)
+    files = {"model-00001-of-00002.safetensors": keys[: len(keys) // 2], "model-00002-of-00002.safetensors": keys[len(keys) // 2:]}
+    wm = {}
+    for fn, ks in files.items():
+        save_file({k: tensors[k].contiguous() for k in ks}, str(src / fn))
+        wm.update({k: fn for k in ks})
+    json.dump({"metadata": {}, "weight_map": wm}, open(src / "model.safetensors.index.json", "w"))
+    json.dump({"hidden_size": 64, "quantization_config": {"quant_method": "fp8"}}, open(src / "config.json", "w"))
+    (src / "tokenizer.json").write_text("{}")
+    blobs = {}
+    for name in qnames:
+        W = tensors[name + ".weight"]
+        s, z, _ = O.quantization_grid(W.float(), 128, 4, torch.bfloat16)
+        q = torch.randint(0, 16, (R, C), generator=g, dtype=torch.uint8)
+        blobs[name] = {"qweight": q, "scale": s, "zero": z}
+        os.makedirs(qdir / name)
+        torch.save(blobs[name], qdir / name / "quantized_weight.pt")
+    block_driver.save_metadata(str(qdir), 4, 128, True)
+    P.main(["--model_name_or_path", str(src), "--quantized_model_path", str(qdir), "--packed_model_path", str(pdir),
+            "--dtype", "bfloat16"])
+    out_wm = json.load(open(pdir / "model.safetensors.index.json"))["weight_map"]
+    shards = sorted(set(out_wm.values()))
+    assert shards == [f"model-{i:05}-of-00004.safetensors" for i in range(1, 5)]
+    back = {}
+    for fn in shards:
+        back.update(load_file(str(pdir / fn)))
+    assert set(back) == set(out_wm)
+    assert out_wm["model.embed_tokens.weight"] == shards[0] and out_wm["lm_head.weight"] == shards[3]
+    assert out_wm["model.norm.weight"] == shards[3] and out_wm["model.layers.0.input_layernorm.weight"] == shards[1]
+    for name in qnames:
+        assert name + ".weight" not in back
+        words, shape = back[name + ".weight_packed"], back[name + ".weight_shape"]
+        assert shape.tolist() == [R, C]
+        assert torch.equal(O.unpack_from_int32(words, 4, [R, C]), blobs[name]["qweight"].to(torch.int8) - 8)
+        assert torch.equal(back[name + ".weight_scale"], blobs[name]["scale"])
+    assert fp8_name + ".weight_scale_inv" not in back
+    rows, cols = torch.arange(R) // 128, torch.arange(C) // 128
+    want = w8.to(torch.bfloat16) * s8.to(torch.bfloat16)[rows][:, cols]  # src/quant_utils.py:267-284 in bf16
+    assert back[fp8_name + ".weight"].dtype == torch.bfloat16 and torch.equal(back[fp8_name + ".weight"], want)
+    for k in ("model.embed_tokens.weight", "lm_head.weight", "model.layers.0.input_layernorm.weight"):
+        assert torch.equal(back[k], tensors[k])
+    cfg = json.load(open(pdir / "config.json"))
+    assert cfg["hidden_size"] == 64 and cfg["quantization_config"]["format"] == "pack-quantized"
+    assert cfg["quantization_config"]["config_groups"]["group_0"]["weights"]["group_size"] == 128
+    assert "re:.*self_attn.*" in cfg["quantization_config"]["ignore"]
+    assert (pdir / "tokenizer.json").exists()
