@@ -7,7 +7,8 @@
  *   - return value: 0 = launched, <0 = MQ_ERR_* (nothing launched, or launching stopped at the failing
  *     kernel); numerical trouble is reported through a device-side `info` word, LAPACK style;
  *   - matrices are row-major, `ld*` are leading dimensions in ELEMENTS;
- *   - no exceptions cross the boundary; calls are re-entrant per stream.
+ *   - no exceptions cross the boundary; calls are re-entrant per stream and may come from several host threads
+ *     (one-time set-up inside the library is guarded).
  *
  * Citations name the MoE-Quant code each entry point replaces (paths relative to that repository).
  */
@@ -26,7 +27,7 @@ extern "C" {
 #define MQ_ERR_LAUNCH (-2)
 #define MQ_ERR_WORKSPACE (-3)
 
-/* element types for `w_dtype` / `round_dtype` */
+/* element types for `x_dtype` / `w_dtype` / `round_dtype` */
 #define MQ_DT_F32 0 /* round_dtype: no rounding */
 #define MQ_DT_BF16 1
 #define MQ_DT_F16 2
@@ -36,20 +37,33 @@ extern "C" {
  * the `input.float()` up-cast in GPTQ.update, src/gptq.py:97-103.
  *   H  : C x C fp32 (ldh).  Only the upper triangle of the old H is read.  The upper triangle is always
  *        written; with mirror != 0 the lower triangle is written too (symmetric copy).
- *   X  : n x C bf16 (ldx), C and ldx even, X 4-byte aligned.   n == 0 just scales H by beta.
+ *   X  : n x C tokens (ldx) of type x_dtype, as the forward hook delivers them (quant.py:79-81 lets the model
+ *        run in float16, bfloat16 or float32):
+ *          MQ_DT_BF16 / MQ_DT_F16 : read as they are by the 16-bit matrix cores -- the products of two such values
+ *                                   are exact in fp32, the same terms the reference sums after its up-cast;
+ *                                   C and ldx even, X 4-byte aligned;
+ *          MQ_DT_F32              : upper tiles of the fp32 GEMM core (fp32-accurate products), no workspace.
+ *        n == 0 just scales H by beta.
  *   workspace: mq_hessian_syrk_workspace_bytes(n, C) bytes (0 when the tile count alone fills the GPU).
+ * mq_hessian_syrk_bf16 is the same call with x_dtype = MQ_DT_BF16.
  */
 size_t mq_hessian_syrk_workspace_bytes(int n, int C);
+int mq_hessian_syrk(float* H, long ldh, const void* X, int x_dtype, long ldx, int n, int C, float beta, float alpha,
+                    int mirror, void* workspace, size_t workspace_bytes, void* stream);
 int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
                          int mirror, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The same accumulation for `groups` independent Hessians of one width C in one call (the experts of an MoE
  * block: the reference loops over forward hooks, one addmm_ per expert, src/gptq.py:97-103 via quant.py:258-277).
  * H, ldh, X, ldx, n, beta, alpha are HOST arrays with one entry per problem; the device pointers they hold follow
- * the rules above.  When every problem has n >= 256 tokens and 16-byte aligned rows, up to 16 problems share a
- * launch and no workspace is touched; otherwise each problem runs as a plain mq_hessian_syrk_bf16 call with the
- * given workspace (mq_hessian_syrk_grouped_workspace_bytes = the largest single requirement). */
+ * the rules above; all X share x_dtype.  When every problem has 16-bit tokens, n >= 256 of them and 16-byte aligned
+ * rows, up to 16 problems share a launch and no workspace is touched; otherwise each problem runs as a plain
+ * mq_hessian_syrk call with the given workspace (mq_hessian_syrk_grouped_workspace_bytes = the largest single
+ * requirement).  mq_hessian_syrk_bf16_grouped is the same call with x_dtype = MQ_DT_BF16. */
 size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C);
+int mq_hessian_syrk_grouped(int groups, float* const* H, const long* ldh, const void* const* X, int x_dtype,
+                            const long* ldx, const int* n, int C, const float* beta, const float* alpha, int mirror,
+                            void* workspace, size_t workspace_bytes, void* stream);
 int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, const void* const* X, const long* ldx,
                                  const int* n, int C, const float* beta, const float* alpha, int mirror, void* workspace,
                                  size_t workspace_bytes, void* stream);

@@ -16,8 +16,10 @@ _vp, _i, _l, _f, _sz = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_size_t
 # name -> (restype, argtypes); mirrors include/moequant_hip.h declaration by declaration
 SIGNATURES = {
     "mq_hessian_syrk_workspace_bytes": (_sz, [_i, _i]),
+    "mq_hessian_syrk": (_i, [_vp, _l, _vp, _i, _l, _i, _i, _f, _f, _i, _vp, _sz, _vp]),
     "mq_hessian_syrk_bf16": (_i, [_vp, _l, _vp, _l, _i, _i, _f, _f, _i, _vp, _sz, _vp]),
     "mq_hessian_syrk_grouped_workspace_bytes": (_sz, [_i, _vp, _i]),
+    "mq_hessian_syrk_grouped": (_i, [_i, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _sz, _vp]),
     "mq_hessian_syrk_bf16_grouped": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _sz, _vp]),
     "mq_symmetrize_upper": (_i, [_vp, _l, _i, _vp]),
     "mq_hessian_prestep": (_i, [_vp, _l, _i, _i, _vp, _vp, _vp]),

@@ -7,6 +7,10 @@
 #define MQ_ERR_ARG (-1)       // bad pointer / size / alignment
 #define MQ_ERR_LAUNCH (-2)    // hipGetLastError() after a launch was not hipSuccess
 #define MQ_ERR_WORKSPACE (-3) // workspace too small
+// element types of weights, activations and rounding targets
+#define MQ_DT_F32 0
+#define MQ_DT_BF16 1
+#define MQ_DT_F16 2
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));

@@ -22,6 +22,7 @@
 //     launch: the (1/3)C^3 flop of the inverse fill the CUs the late elimination steps leave idle.
 //   finalize: U[j, k] /= U[j, j], strictly lower part zeroed.
 #include <cstdlib>
+#include <mutex>
 
 #include "gemm_f32_tile.hpp"
 
@@ -535,8 +536,8 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
   if (!S || !A || !info || C <= 0 || ld < C || lds < C) return MQ_ERR_ARG;
   if (C % NB != 0) return MQ_ERR_ARG;  // the host pads with an identity block
   hipStream_t st = (hipStream_t)stream;
-  static bool attr_done = false;
-  if (!attr_done) {
+  static std::once_flag once;  // kernel attributes and tuning knobs: set once, whichever host thread comes first
+  std::call_once(once, [] {
     if (const char* e = getenv("MQ_INV_KC")) INV_KC = atoi(e) > 0 ? atoi(e) : INV_KC;
     if (const char* e = getenv("MQ_PANELS")) TRAIL_PANELS = atoi(e) > 0 ? atoi(e) : TRAIL_PANELS;
     (void)hipFuncSetAttribute((const void*)revchol_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -547,8 +548,7 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
                               (int)gemmf32::short_smem_bytes(2));
     (void)hipFuncSetAttribute((const void*)inv_first_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)gemmf32::SMEM_BYTES);
-    attr_done = true;
-  }
+  });
   if ((ld & 3) || ((uintptr_t)A & 15) || (lds & 3) || ((uintptr_t)S & 15)) return MQ_ERR_ARG;  // float4 access to rows
   int rc;
   auto kc_of = [&](int) { return INV_KC; };  // one depth for all block rows: 2, 3 for the short rows measured no faster

@@ -3,6 +3,8 @@
 // so every fragment read is a conflict-free ds_read_b32 whatever the global layout was.
 // Used by the factorisation (trailing update, panel solve, triangular inverse) and by the
 // GPTQ lazy-batch trailing update.
+#include <mutex>
+
 #include "gemm_f32_tile.hpp"
 
 namespace {
@@ -26,12 +28,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 
 template <bool A_KC, bool B_KC>
 int launch(const GemmF32& g, int tiles_n, int total, int vecA, int vecB, int pair_rows, hipStream_t stream) {
-  static bool attr_done = false;
-  if (!attr_done) {
+  static std::once_flag once;
+  std::call_once(once, [] {
     (void)hipFuncSetAttribute((const void*)gemm_f32_kernel<A_KC, B_KC>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)SMEM_BYTES);
-    attr_done = true;
-  }
+  });
   hipLaunchKernelGGL((gemm_f32_kernel<A_KC, B_KC>), dim3(total, 1, g.batch), dim3(256), SMEM_BYTES, stream, g, tiles_n,
                      total, vecA, vecB, pair_rows);
   return mq_check_launch();

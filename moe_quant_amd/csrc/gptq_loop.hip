@@ -19,6 +19,9 @@
 // y = round_to(dtype)((q - z) * s), e = y - x, w_k = fma(U[j,k], e, w_k).
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
+#include <mutex>
+
 #include "gemm_f32_tile.hpp"
 
 namespace {
@@ -432,8 +435,8 @@ constexpr size_t BLOCK_SMEM = COL_SMEM > gemmf32::SMEM_BYTES ? COL_SMEM : gemmf3
 template <bool ROWMAP, bool QZERO>
 int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   const int grid = (a.R + 63) / 64;
-  static bool attr_done = false;
-  if (!attr_done) {
+  static std::once_flag once;  // one per template instance
+  std::call_once(once, [] {
     (void)hipFuncSetAttribute((const void*)gptq_block_kernel<true, ROWMAP, QZERO>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
     (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO>,
@@ -442,8 +445,7 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
       const int v = atoi(e);
       if (v >= 1 && v <= LOOP_BATCH_MAX) LOOP_BATCH = v;
     }
-    attr_done = true;
-  }
+  });
   LoopArgs la = a;
   int blk = 0, nbprev = 0;
   for (int i1 = 0; i1 < a.C; i1 += block, ++blk) {

@@ -9,6 +9,8 @@
 //
 // flags (int32[4], device): [0] NaN found (H was replaced by the identity), [1] number of pruned channels,
 // [2] number of cleared channels (pruned or all-zero weights), [3] unused.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace {

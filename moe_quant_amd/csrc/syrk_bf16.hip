@@ -1,8 +1,10 @@
-// Hessian accumulation  H <- beta*H + alpha * X^T X  for bf16 activations X (n x C, row-major) and an
-// fp32 Hessian, on the bf16 matrix cores of gfx950 (v_mfma_f32_32x32x16_bf16).
+// Hessian accumulation  H <- beta*H + alpha * X^T X  for 16-bit activations X (n x C, row-major; bf16 or
+// fp16) and an fp32 Hessian, on the 16-bit matrix cores of gfx950 (v_mfma_f32_32x32x16_bf16 / _f16).
 //
-// bf16*bf16 products are exact in fp32, so reading the bf16 tokens directly gives the same terms as
-// up-casting X to fp32 first; only the summation order differs.
+// bf16*bf16 and fp16*fp16 products are exact in fp32 (8+8 and 11+11 significand bits), so reading the
+// 16-bit tokens directly gives the same terms as up-casting X to fp32 first; only the summation order
+// differs.  Data movement is the same for both types: only the matrix instruction changes (template flag F16).
+// fp32 activations go through the fp32 GEMM tiles instead (see mq_hessian_syrk).
 //
 // Only tiles of the upper block triangle are computed.  X is token-major, the matrix cores want the
 // reduction index (tokens) contiguous per lane, so every thread loads a 2-channel x 8-token patch with
@@ -10,6 +12,7 @@
 // tile laid out [channel][token].  With too few tiles to fill 256 CUs the token range is split; the
 // partial tiles go to a caller-provided workspace and are reduced in a fixed order (deterministic).
 #include <cstdlib>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -34,6 +37,16 @@ __device__ __forceinline__ void tri_decode(int L, int& tm, int& tn) {
   while ((c + 1) * (c + 2) / 2 <= L) ++c;
   tn = c;
   tm = L - c * (c + 1) / 2;
+}
+
+typedef _Float16 half8n __attribute__((ext_vector_type(8)));
+// one 32x32x16 product on 16-bit operands, fp32 accumulation; the operands travel as bf16x8n bit patterns
+template <bool F16>
+__device__ __forceinline__ floatx16 mfma16(bf16x8n a, bf16x8n b, floatx16 c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8n, a), __builtin_bit_cast(half8n, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
 struct Patch {
@@ -86,6 +99,7 @@ __device__ __forceinline__ void write_tile(float* __restrict__ H, long ldh, int 
   }
 }
 
+template <bool F16>
 __global__ __launch_bounds__(256) void syrk_bf16_kernel(float* __restrict__ H, long ldh, const uint16_t* __restrict__ X,
                                                         long ldx, int n, int C, float alpha, float beta, int ntri,
                                                         int splits, int tokens_per_split, float* __restrict__ ws,
@@ -139,10 +153,10 @@ __global__ __launch_bounds__(256) void syrk_bf16_kernel(float* __restrict__ H, l
       const bf16x8n a1 = *reinterpret_cast<const bf16x8n*>(as + 32 * LDS_ROW + kk * 16);
       const bf16x8n b0 = *reinterpret_cast<const bf16x8n*>(bs + kk * 16);
       const bf16x8n b1 = *reinterpret_cast<const bf16x8n*>(bs + 32 * LDS_ROW + kk * 16);
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
+      acc[0][0] = mfma16<F16>(a0, b0, acc[0][0]);
+      acc[0][1] = mfma16<F16>(a0, b1, acc[0][1]);
+      acc[1][0] = mfma16<F16>(a1, b0, acc[1][0]);
+      acc[1][1] = mfma16<F16>(a1, b1, acc[1][1]);
     }
     if (kt + 1 < nk) {
       uint16_t* nx = tiles + (cur ^ 1) * 2 * TILE_ELEMS;
@@ -465,7 +479,7 @@ __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsign
 // one 256x256 tile (or one token split of it); bid = linear workgroup index among ntri*splits.
 // NW = 4: four wavefronts of 128x128 (one per SIMD, all 512 registers).  NW = 8: eight of 128x64, two per SIMD:
 // while one waits for the address unit to take its direct loads the other keeps the matrix pipe busy.
-template <int NW>
+template <int NW, bool F16>
 __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx,
                                               int n, int C, float alpha, float beta, int ntri, int splits,
                                               int tokens_per_split, float* __restrict__ ws, int bid,
@@ -562,8 +576,7 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8n, va[i]),
-                                                              __builtin_bit_cast(bf16x8n, vb[j]), acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma16<F16>(__builtin_bit_cast(bf16x8n, va[i]), __builtin_bit_cast(bf16x8n, vb[j]), acc[i][j]);
     }
   }
 #undef MQ_SYRK_ISSUE
@@ -595,14 +608,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
     int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  syrk_dma_tile<4>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+  syrk_dma_tile<4, false>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
 }
 
+template <bool F16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_bf16_dma8_kernel(
     float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
     int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  syrk_dma_tile<8>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+  syrk_dma_tile<8, F16>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
 }
 
 // Several independent accumulations (one Hessian each, same C) in one launch: blockIdx.y picks the problem.
@@ -616,12 +630,13 @@ struct SyrkGroupTable {
   int n[SYRK_MAX_GROUP];
   float alpha[SYRK_MAX_GROUP], beta[SYRK_MAX_GROUP];
 };
+template <bool F16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_bf16_dma_grouped_kernel(
     SyrkGroupTable t, int C, int ntri) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int z = blockIdx.y;
   const int tps = (t.n[z] + KT3 - 1) / KT3 * KT3;
-  syrk_dma_tile<8>(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
+  syrk_dma_tile<8, F16>(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
                 smem);
 }
 
@@ -738,34 +753,59 @@ extern "C" int mq_symmetrize_upper(float* H, long ldh, int C, void* stream) {
   return mq_check_launch();
 }
 
-extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
-                                    int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+// fp32 activations: the same accumulation as upper 128x128 tiles of the fp32 GEMM core (gemm_f32_tile.hpp), whose
+// products are fp32-accurate (what `input.float()` followed by addmm_ computes, up to summation order).
+static int syrk_f32(float* H, long ldh, const float* X, long ldx, int n, int C, float beta, float alpha, int mirror,
+                    hipStream_t st) {
+  const float* Xp = X ? X : H;  // n == 0: never dereferenced, the tiles only scale H by beta
+  GemmF32 g{Xp, Xp, H, 1, ldx, ldx, 1, ldh, C, C, n, alpha, beta, 1, 0, 1, 0, 0, 0};
+  const int rc = mq_launch_gemm_f32(g, st);
+  if (rc != MQ_OK) return rc;
+  return mirror ? mq_symmetrize_upper(H, ldh, C, st) : MQ_OK;
+}
+
+extern "C" int mq_hessian_syrk(float* H, long ldh, const void* X, int x_dtype, long ldx, int n, int C, float beta,
+                               float alpha, int mirror, void* workspace, size_t workspace_bytes, void* stream) {
   if (!H || C <= 0 || n < 0 || ldh < C || (n > 0 && (!X || ldx < C))) return MQ_ERR_ARG;
+  if (x_dtype != MQ_DT_F32 && x_dtype != MQ_DT_BF16 && x_dtype != MQ_DT_F16) return MQ_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (x_dtype == MQ_DT_F32) {
+    if ((uintptr_t)X & 3) return MQ_ERR_ARG;
+    return syrk_f32(H, ldh, (const float*)X, ldx, n, C, beta, alpha, mirror, st);
+  }
+  const bool f16 = x_dtype == MQ_DT_F16;
   if ((C & 1) || (ldx & 1) || ((uintptr_t)X & 3)) return MQ_ERR_ARG;  // 4-byte channel-pair loads
   int ntri, splits, tps;
-  hipStream_t st = (hipStream_t)stream;
+  static std::once_flag once;
+  static bool use_dma = true;
+  static int dma_waves = 8;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)BIG_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)DMA_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)DMA_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)DMA_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)SMEM_BYTES);
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)SMEM_BYTES);
+    (void)hipFuncSetAttribute((const void*)syrk_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);
+    use_dma = getenv("MQ_SYRK_OLD") == nullptr;
+    dma_waves = getenv("MQ_SYRK_W4") ? 4 : 8;  // the one-wavefront-per-SIMD kernel stays for comparison (bf16 only)
+  });
   if (n > 0 && use_big(X, ldx, n, C)) {
     pick_split_big(n, C, ntri, splits, tps);
     if (splits > 1) {
       const size_t need = (size_t)splits * ntri * T2 * T2 * sizeof(float);
       if (!workspace || workspace_bytes < need) return MQ_ERR_WORKSPACE;
     }
-    static bool big_attr = false;
-    static bool use_dma = true;
-    if (!big_attr) {
-      (void)hipFuncSetAttribute((const void*)syrk_bf16_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)BIG_SMEM);
-      (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)DMA_SMEM);
-      (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)DMA_SMEM);
-      use_dma = getenv("MQ_SYRK_OLD") == nullptr;
-      big_attr = true;
-    }
-    static const int dma_waves = getenv("MQ_SYRK_W4") ? 4 : 8;  // the one-wavefront-per-SIMD kernel stays for comparison
-    if (use_dma && dma_waves == 8)
-      hipLaunchKernelGGL(syrk_bf16_dma8_kernel, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
-                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    if (f16)
+      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<true>, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh,
+                         (const uint16_t*)X, ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+    else if (use_dma && dma_waves == 8)
+      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<false>, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh,
+                         (const uint16_t*)X, ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
     else if (use_dma)
       hipLaunchKernelGGL(syrk_bf16_dma_kernel, dim3(ntri * splits), dim3(256), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
                          ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
@@ -782,18 +822,16 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
     return mirror ? mq_symmetrize_upper(H, ldh, C, stream) : MQ_OK;
   }
   pick_split(n > 0 ? n : 1, C, ntri, splits, tps);
-  static bool attr_done = false;
-  if (!attr_done) {
-    (void)hipFuncSetAttribute((const void*)syrk_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);
-    (void)hipFuncSetAttribute((const void*)syrk_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);
-    attr_done = true;
-  }
   if (splits > 1) {
     const size_t need = (size_t)splits * ntri * T * T * sizeof(float);
     if (!workspace || workspace_bytes < need) return MQ_ERR_WORKSPACE;
   }
-  hipLaunchKernelGGL(syrk_bf16_kernel, dim3(ntri * splits), dim3(256), SMEM_BYTES, st, H, ldh, (const uint16_t*)X, ldx,
-                     n, C, alpha, beta, ntri, splits, tps, (float*)workspace, mirror);
+  if (f16)
+    hipLaunchKernelGGL(syrk_bf16_kernel<true>, dim3(ntri * splits), dim3(256), SMEM_BYTES, st, H, ldh, (const uint16_t*)X,
+                       ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace, mirror);
+  else
+    hipLaunchKernelGGL(syrk_bf16_kernel<false>, dim3(ntri * splits), dim3(256), SMEM_BYTES, st, H, ldh, (const uint16_t*)X,
+                       ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace, mirror);
   int rc = mq_check_launch();
   if (rc != MQ_OK) return rc;
   if (splits > 1) {
@@ -804,8 +842,14 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
   return rc;
 }
 
+extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int C, float beta, float alpha,
+                                    int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+  return mq_hessian_syrk(H, ldh, X, MQ_DT_BF16, ldx, n, C, beta, alpha, mirror, workspace, workspace_bytes, stream);
+}
+
 // Host arrays of `groups` entries each.  Problems that the direct-load kernel cannot take (few tokens, unaligned
-// rows) make the whole call fall back to one plain call per problem, so the result never depends on the path.
+// rows, fp32 tokens) make the whole call fall back to one plain call per problem, so the result never depends on
+// the path.
 extern "C" size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C) {
   size_t need = 0;
   for (int g = 0; g < groups; ++g) {
@@ -815,11 +859,12 @@ extern "C" size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int*
   return need;
 }
 
-extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, const void* const* X,
-                                            const long* ldx, const int* n, int C, const float* beta, const float* alpha,
-                                            int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int mq_hessian_syrk_grouped(int groups, float* const* H, const long* ldh, const void* const* X, int x_dtype,
+                                       const long* ldx, const int* n, int C, const float* beta, const float* alpha,
+                                       int mirror, void* workspace, size_t workspace_bytes, void* stream) {
   if (groups < 0 || C <= 0 || (groups > 0 && (!H || !ldh || !X || !ldx || !n || !beta || !alpha))) return MQ_ERR_ARG;
-  bool fast = groups > 1;
+  if (x_dtype != MQ_DT_F32 && x_dtype != MQ_DT_BF16 && x_dtype != MQ_DT_F16) return MQ_ERR_ARG;
+  bool fast = groups > 1 && x_dtype != MQ_DT_F32;
   for (int g = 0; g < groups; ++g) {
     if (!H[g] || n[g] < 0 || ldh[g] < C || (n[g] > 0 && (!X[g] || ldx[g] < C))) return MQ_ERR_ARG;
     if (n[g] <= 0 || !use_big(X[g], ldx[g], n[g], C)) fast = false;
@@ -827,18 +872,19 @@ extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const l
   hipStream_t st = (hipStream_t)stream;
   if (!fast) {
     for (int g = 0; g < groups; ++g) {
-      const int rc = mq_hessian_syrk_bf16(H[g], ldh[g], X[g], ldx[g], n[g], C, beta[g], alpha[g], mirror, workspace,
-                                          workspace_bytes, stream);
+      const int rc = mq_hessian_syrk(H[g], ldh[g], X[g], x_dtype, ldx[g], n[g], C, beta[g], alpha[g], mirror, workspace,
+                                     workspace_bytes, stream);
       if (rc != MQ_OK) return rc;
     }
     return MQ_OK;
   }
-  static bool attr_done = false;
-  if (!attr_done) {
-    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_grouped_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+  static std::once_flag once;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_grouped_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)DMA_SMEM);
-    attr_done = true;
-  }
+    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_grouped_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)DMA_SMEM);
+  });
   const int tiles = (C + T2 - 1) / T2, ntri = tiles * (tiles + 1) / 2;
   for (int g0 = 0; g0 < groups; g0 += SYRK_MAX_GROUP) {
     const int cnt = groups - g0 < SYRK_MAX_GROUP ? groups - g0 : SYRK_MAX_GROUP;
@@ -853,7 +899,10 @@ extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const l
       t.alpha[i] = alpha[g];
       t.beta[i] = beta[g];
     }
-    hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel, dim3(ntri, cnt), dim3(512), DMA_SMEM, st, t, C, ntri);
+    if (x_dtype == MQ_DT_F16)
+      hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel<true>, dim3(ntri, cnt), dim3(512), DMA_SMEM, st, t, C, ntri);
+    else
+      hipLaunchKernelGGL(syrk_bf16_dma_grouped_kernel<false>, dim3(ntri, cnt), dim3(512), DMA_SMEM, st, t, C, ntri);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     if (mirror)
@@ -861,4 +910,11 @@ extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const l
         if ((rc = mq_symmetrize_upper(H[g0 + i], ldh[g0 + i], C, stream)) != MQ_OK) return rc;
   }
   return MQ_OK;
+}
+
+extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, const void* const* X,
+                                            const long* ldx, const int* n, int C, const float* beta, const float* alpha,
+                                            int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+  return mq_hessian_syrk_grouped(groups, H, ldh, X, MQ_DT_BF16, ldx, n, C, beta, alpha, mirror, workspace, workspace_bytes,
+                                 stream);
 }

@@ -1,9 +1,10 @@
 """Drop-in for MoE-Quant's src/gptq.py: the same `GPTQ` handle, its numeric work done by HIP kernels.
 
-Out of scope (raise instead of silently differing): asymmetric grids, conv layers, the MSE scale
-search, the multi-GPU Hessian all-reduce.  Inputs to `update` must be bf16 (the engine's SYRK reads
-bf16 tokens directly; bf16 x bf16 products are exact in fp32, so nothing is lost versus the
-reference's up-cast to fp32)."""
+Out of scope (raise instead of silently differing): asymmetric grids, conv layers, the multi-GPU
+Hessian all-reduce.  `update` takes bf16, fp16 or fp32 activations, the dtypes the reference's driver
+offers (quant.py:79-81): 16-bit tokens are read as they are by the matrix cores (their pairwise
+products are exact in fp32, so nothing is lost versus the reference's up-cast, src/gptq.py:97), fp32
+tokens go through fp32-accurate GEMM tiles.  `quantization_scale="mse"` runs the scale search."""
 from __future__ import annotations
 
 import warnings
@@ -18,6 +19,9 @@ from torch import Tensor
 from . import linalg_utils, ops
 
 
+_ACT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+
+
 class QuantizationOrder(Enum):
     DEFAULT = "default"
     ACTIVATION = "activation"
@@ -25,6 +29,8 @@ class QuantizationOrder(Enum):
 
 class GPTQ:
     """Mirror of src/gptq.py:22-243 (constructor arguments, attributes and methods keep their names)."""
+
+    factor_calls = 0  # factorisations computed so far by all handles (a tied handle that reuses its owner's adds none)
 
     def __init__(
         self,
@@ -129,13 +135,15 @@ class GPTQ:
     @torch.no_grad()
     def update(self, input: Tensor) -> None:
         input = input.reshape(-1, input.shape[-1])
-        if input.dtype != torch.bfloat16:
-            raise TypeError(f"GPTQ.update needs bf16 activations, got {input.dtype}")
+        if input.dtype not in _ACT_DTYPES:
+            raise TypeError(f"GPTQ.update takes bf16, fp16 or fp32 activations, got {input.dtype}")
         num_new_samples = input.shape[0]
         if num_new_samples == 0:
-            if self.H is None:
-                self.H = torch.zeros((self.d_col, self.d_col), device=input.device, dtype=torch.float32)
-            return  # the reference would divide 0/0 here when nothing was collected before
+            # Nothing to add (an expert that received no token in this batch).  With samples collected before,
+            # the reference's update is the identity (beta = 1, alpha * 0); with none it divides 0/0.  Either way
+            # H is left as it is: a handle that never sees a token keeps H = None and takes the pre-step's
+            # identity / issue_zero_samples path, exactly like a handle whose hook never fired.
+            return
         if self.H is None:
             # the first product runs with beta = 0 and writes the whole upper triangle, the pre-step mirrors it:
             # no need to clear 4*C^2 bytes first
@@ -159,8 +167,8 @@ class GPTQ:
         Hs, Xs, betas, alphas = [], [], [], []
         for h, x in zip(handles, inputs):
             x = x.reshape(-1, x.shape[-1])
-            if x.dtype != torch.bfloat16:
-                raise TypeError(f"GPTQ.update needs bf16 activations, got {x.dtype}")
+            if x.dtype not in _ACT_DTYPES:
+                raise TypeError(f"GPTQ.update takes bf16, fp16 or fp32 activations, got {x.dtype}")
             if x.shape[0] == 0:
                 continue
             if h.H is None:
@@ -291,7 +299,20 @@ class GPTQ:
 
     def quantize(self, bits: int | float) -> Tuple[Tensor, Tensor, Tensor]:
         self.quantization_pre_step()
+        self._pin_inputs_to_current_stream()
         return self._quantize(bits)
+
+    def _pin_inputs_to_current_stream(self) -> None:
+        """The layer's weight and H were allocated on whatever stream loaded the model / ran the hooks; a caller may
+        run `quantize` on another stream and drop its last reference to either (`layer.weight.data = ...`,
+        `handle.H = None`) while this stream's kernels are still queued.  Telling the caching allocator that this
+        stream uses them keeps it from handing their memory to a new tensor before those kernels have run."""
+        if not self.W_device.type == "cuda":
+            return
+        cur = torch.cuda.current_stream(self.W_device)
+        for t in (self.layer.weight, self.H):
+            if isinstance(t, Tensor) and t.is_cuda:
+                t.record_stream(cur)
 
     def packed_words(self) -> Tensor:
         """int32 (R, C/8) compressed_tensors words of the last `quantize` call, packed straight from the
@@ -314,6 +335,7 @@ class GPTQ:
         # a failed factorisation yields the identity on the device, the reference's `except` branch
         # (src/gptq.py:239-240, which never sets issue_non_invertible; this engine does)
         U, self._info = linalg_utils.inverse_cholesky_factor(H)
+        GPTQ.factor_calls += 1
         if self.num_tied_handles > 0:
             self._hessian_inv = U
         return U

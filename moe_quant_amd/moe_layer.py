@@ -35,7 +35,10 @@ class LayerResult:
     scales: Dict[str, torch.Tensor] = field(default_factory=dict)
     qweight: Dict[str, torch.Tensor] = field(default_factory=dict)  # only for the experts listed in keep_codes
     hessians: Dict[str, torch.Tensor] = field(default_factory=dict)  # idem (undamped copies)
+    down_inputs: Dict[int, torch.Tensor] = field(default_factory=dict)  # idem: what the expert's down_proj saw
     issues: Dict[str, int] = field(default_factory=dict)
+    issues_by_linear: Dict[str, List[str]] = field(default_factory=dict)  # "<e>.<proj>" -> names of raised flags
+    factorizations: int = 0  # Hessian factorisations actually computed (a tied up_proj reuses its gate_proj's)
 
 
 def route_tokens(expert_ids: torch.Tensor, n_experts: int):
@@ -103,6 +106,9 @@ def quantize_moe_layer(
             g.update(xe)
             a = torch.nn.functional.silu(xe @ experts[e].gate.t()) * (xe @ experts[e].up.t())  # the expert's forward
             d.update(a)
+            if e in keep_codes:
+                prev = res.down_inputs.get(e)
+                res.down_inputs[e] = a if prev is None else torch.cat([prev, a])
     sync()
     res.seconds["hessians_incl_gather_and_forward"] = time.perf_counter() - t1
 
@@ -113,7 +119,8 @@ def quantize_moe_layer(
     for s_ in lanes:
         if s_ is not main:
             s_.wait_stream(main)
-    done = []  # handles whose verdict words are read after everything is queued
+    done = []  # (name, handle): verdict words are read after everything is queued
+    factor_calls_before = GPTQ.factor_calls
     for e, (g, u, d) in enumerate(handles):
         lane = lanes[e % len(lanes)]
         with torch.cuda.stream(lane):
@@ -127,7 +134,7 @@ def quantize_moe_layer(
             for name, h in (("gate_proj", g), ("up_proj", u), ("down_proj", d)):
                 q, s, z = h.quantize(bits)
                 words = h.packed_words()
-                done.append(h)
+                done.append((f"{e}.{name}", h))
                 if keep_outputs:
                     res.packed[f"{e}.{name}"] = words
                     res.scales[f"{e}.{name}"] = s
@@ -146,10 +153,14 @@ def quantize_moe_layer(
             main.wait_stream(s_)
     sync()
     issues = {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
-    for h in done:
-        issues["zero_samples"] += int(h.issue_zero_samples)
-        issues["nan_hessian"] += int(h.issue_nan_hessian)
-        issues["non_invertible"] += int(h.issue_non_invertible)
+    for name, h in done:
+        raised = [k for k, v in (("zero_samples", h.issue_zero_samples), ("nan_hessian", h.issue_nan_hessian),
+                                 ("non_invertible", h.issue_non_invertible)) if v]
+        for k in raised:
+            issues[k] += 1
+        if raised:
+            res.issues_by_linear[name] = raised
+    res.factorizations = GPTQ.factor_calls - factor_calls_before
     res.seconds["quantize_and_pack"] = time.perf_counter() - t2
     res.seconds["total"] = time.perf_counter() - t0
     res.issues = issues

@@ -56,25 +56,25 @@ _ws = _Workspace()
 
 # ---- (1) Hessian ------------------------------------------------------------------------------------
 def hessian_syrk_(H: Tensor, X: Tensor, beta: float, alpha: float, mirror: bool = True) -> Tensor:
-    """H <- beta*H + alpha*X^T X in place.  H (C,C) fp32, X (n,C) bf16, rows may be strided."""
+    """H <- beta*H + alpha*X^T X in place.  H (C,C) fp32, X (n,C) bf16, fp16 or fp32, rows may be strided."""
     _dev(H, X)
     lib = _lib.load()
     C = H.shape[0]
     if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
         raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
-    if X.dtype != torch.bfloat16 or X.dim() != 2 or X.shape[1] != C:
-        raise ValueError("X must be (n,C) bf16")
+    if X.dtype not in _DT or X.dim() != 2 or X.shape[1] != C:
+        raise ValueError("X must be (n,C) bf16, fp16 or fp32")
     if X.shape[0] > 0 and X.stride(1) != 1:
         X = X.contiguous()
     n = X.shape[0]
-    need = lib.mq_hessian_syrk_workspace_bytes(n, C)
+    need = lib.mq_hessian_syrk_workspace_bytes(n, C) if X.dtype != torch.float32 else 0
     ws = _ws.get(H.device, need, "syrk") if need else None
     ldx = X.stride(0) if n > 1 else C
-    rc = lib.mq_hessian_syrk_bf16(
-        H.data_ptr(), H.stride(0), X.data_ptr() if n else None, ldx, n, C, beta, alpha, int(mirror),
+    rc = lib.mq_hessian_syrk(
+        H.data_ptr(), H.stride(0), X.data_ptr() if n else None, _DT[X.dtype], ldx, n, C, beta, alpha, int(mirror),
         _p(ws), need, _stream(H),
     )
-    check(rc, "mq_hessian_syrk_bf16")
+    check(rc, "mq_hessian_syrk")
     return H
 
 
@@ -91,11 +91,12 @@ def hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror: bool = True) -> None:
     _dev(*Hs, *Xs)
     C = Hs[0].shape[0]
     Xs = [x if (x.shape[0] == 0 or x.stride(1) == 1) else x.contiguous() for x in Xs]
+    xdt = Xs[0].dtype
     for H, X in zip(Hs, Xs):
         if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
             raise ValueError("every H must be a (C,C) fp32 matrix with unit column stride")
-        if X.dtype != torch.bfloat16 or X.dim() != 2 or X.shape[1] != C:
-            raise ValueError("every X must be (n,C) bf16")
+        if X.dtype not in _DT or X.dtype != xdt or X.dim() != 2 or X.shape[1] != C:
+            raise ValueError("every X must be (n,C), all of one type (bf16, fp16 or fp32)")
     ns = (C_.c_int * k)(*[x.shape[0] for x in Xs])
     Hp = (C_.c_void_p * k)(*[h.data_ptr() for h in Hs])
     Xp = (C_.c_void_p * k)(*[(x.data_ptr() if x.shape[0] else None) for x in Xs])
@@ -105,8 +106,9 @@ def hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror: bool = True) -> None:
     al = (C_.c_float * k)(*[float(a) for a in alphas])
     need = lib.mq_hessian_syrk_grouped_workspace_bytes(k, ns, C)
     ws = _ws.get(Hs[0].device, need, "syrk") if need else None
-    rc = lib.mq_hessian_syrk_bf16_grouped(k, Hp, ldh, Xp, ldx, ns, C, be, al, int(mirror), _p(ws), need, _stream(Hs[0]))
-    check(rc, "mq_hessian_syrk_bf16_grouped")
+    rc = lib.mq_hessian_syrk_grouped(k, Hp, ldh, Xp, _DT[xdt], ldx, ns, C, be, al, int(mirror), _p(ws), need,
+                                     _stream(Hs[0]))
+    check(rc, "mq_hessian_syrk_grouped")
 
 
 def symmetrize_upper_(H: Tensor) -> Tensor:

@@ -23,7 +23,7 @@ def _declared():
 
 def test_header_declares_the_expected_entry_points():
     d = _declared()
-    for name in ("mq_hessian_syrk_bf16", "mq_factor_upper_inverse", "mq_quant_grid_sym", "mq_prepare_wt",
+    for name in ("mq_hessian_syrk", "mq_hessian_syrk_grouped", "mq_hessian_syrk_bf16", "mq_factor_upper_inverse", "mq_quant_grid_sym", "mq_prepare_wt",
                  "mq_gptq_loop", "mq_untranspose_codes", "mq_pack_int4", "mq_pack_from_qt", "mq_gemm_f32",
                  "mq_hessian_syrk_workspace_bytes"):
         assert name in d
@@ -123,7 +123,9 @@ def test_handle_surface_matches_reference():
     # reset(): it drops its own reference and never decrements the owner's counter
     assert tied.H is None and owner.num_tied_handles == 1 and owner.H is not None
     with pytest.raises(TypeError):
-        h.update(torch.zeros(4, 256))  # fp32 activations are refused, not silently down-cast
+        h.update(torch.zeros(4, 256, dtype=torch.float64))  # only the reference driver's dtypes: fp16, bf16, fp32
+    h.update(torch.zeros(0, 256))  # an empty batch is a no-op (and touches no kernel)
+    assert h.H is None and h.tokens_collected == 0
 
 
 def test_reference_module_names_resolve():

@@ -237,3 +237,42 @@ def test_pack_command_line_on_a_synthetic_checkpoint(dev, tmp_path):
     assert cfg["quantization_config"]["config_groups"]["group_0"]["weights"]["group_size"] == 128
     assert "re:.*self_attn.*" in cfg["quantization_config"]["ignore"]
     assert (pdir / "tokenizer.json").exists()
+
+
+def test_mixed_size_linears_on_three_lanes_equal_one_lane(dev):
+    """Linears of very different cost on three lanes (the lanes drift apart) while the driver swaps weights and
+    drops Hessians behind the queued kernels: codes, scales and the replaced weights must be bit-identical to the
+    one-lane run of the same block."""
+    sizes = [(128, 1536), (1024, 256), (256, 128), (128, 1024), (640, 384), (128, 2048), (512, 128), (256, 896)]
+
+    class Bag(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.ModuleList([nn.Linear(c, r, bias=False) for r, c in sizes])
+
+    def run(streams):
+        torch.manual_seed(3)
+        bag = Bag().to(dev).to(torch.bfloat16)
+        g = torch.Generator().manual_seed(4)
+        xs = [torch.randn(700, c, generator=g).to(torch.bfloat16).to(dev) for _, c in sizes]
+
+        def fwd():
+            for lin, x in zip(bag.lin, xs):
+                lin(x)
+
+        import tempfile
+
+        with tempfile.TemporaryDirectory() as d:
+            block_driver.quantize_block(bag, "lin.", fwd, bits=4, group_size=128, save_dir=d, streams=streams)
+            blobs = {n: torch.load(os.path.join(d, n, "quantized_weight.pt"), weights_only=True) for n in os.listdir(d)}
+        return blobs, [lin.weight.data.clone() for lin in bag.lin]
+
+    b1, w1 = run(1)
+    for rep in range(3):
+        b3, w3 = run(3)
+        assert set(b1) == set(b3) and len(b1) == len(sizes)
+        for n in b1:
+            for k in ("qweight", "scale", "zero"):
+                assert torch.equal(b1[n][k], b3[n][k]), (rep, n, k)
+        for a, b in zip(w1, w3):
+            assert torch.equal(a, b)

@@ -169,6 +169,40 @@ def test_zero_samples_is_round_to_nearest(dev):
     assert torch.equal(q.cpu(), ref["qweight"]) and torch.equal(s.cpu(), ref["scale"])
 
 
+def test_empty_update_only_is_the_zero_samples_path(dev):
+    """A hook that only ever delivers zero tokens (an expert no token was routed to): H stays None, the pre-step
+    takes the identity with issue_zero_samples -- not a zero Hessian that would prune every channel."""
+    W = synth.weight(128, 256, 11)
+    h = GPTQ(_layer(W, dev), 128, True)
+    h.update(torch.zeros(0, 256, dtype=torch.bfloat16, device=dev))
+    GPTQ.update_many([h], [torch.zeros(0, 256, dtype=torch.bfloat16, device=dev)])
+    assert h.H is None and h.tokens_collected == 0
+    q, s, z = h.quantize(4)
+    assert h.issue_zero_samples and not h.issue_nan_hessian
+    ref = O.quantize_linear(W, None)
+    assert torch.equal(q.cpu(), ref["qweight"]) and torch.equal(s.cpu(), ref["scale"])
+    assert not torch.all(q == 8)
+    # and an empty batch after real ones changes nothing
+    h2 = GPTQ(_layer(W, dev), 128, True)
+    X = synth.activations_outlier(300, 256, 12).to(dev)
+    h2.update(X)
+    H_before = h2.H.clone()
+    h2.update(X[:0])
+    assert torch.equal(h2.H, H_before) and h2.tokens_collected == 300
+
+
+@pytest.mark.parametrize("wdt,xdt", [(torch.float16, torch.float16), (torch.bfloat16, torch.float32),
+                                     (torch.float32, torch.float32), (torch.bfloat16, torch.float16)])
+def test_model_dtypes_of_the_reference_driver(dev, wdt, xdt):
+    """quant.py:79-81 offers float16 (its default), bfloat16 and float32 models: weights, activations, scale
+    rounding and the loop's dequantized values follow that dtype, end to end against the oracle."""
+    case = synth.config1(0.125)
+    case.W = case.W.float().to(wdt)
+    case.X = case.X.float().to(xdt)
+    case.name = f"cfg1_eighth_{wdt}_{xdt}"
+    _run_case(case, dev, chunks=2)
+
+
 def test_nan_hessian_falls_back(dev):
     W = synth.weight(64, 256, 2)
     h = GPTQ(_layer(W, dev), 128, True)

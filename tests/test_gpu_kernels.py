@@ -110,10 +110,13 @@ def test_gemm_f32_tri_and_ktrim(dev):
 
 
 # ---------------------------------------------------------------- (1) Hessian SYRK
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("n,C", [(1024, 896), (4096, 256), (100, 128), (33, 384), (5000, 640)])
-def test_hessian_syrk_vs_fp64(dev, n, C):
-    _say(f"syrk n={n} C={C}")
-    X = synth.activations_outlier(n, C, seed=n + C)
+def test_hessian_syrk_vs_fp64(dev, n, C, dtype):
+    """Every activation dtype the reference's driver offers (quant.py:79-81), against the fp64 closed form of the
+    values as stored in that dtype: the 1e-5 relative Frobenius gate."""
+    _say(f"syrk n={n} C={C} {dtype}")
+    X = synth.activations_outlier(n, C, seed=n + C, dtype=dtype)
     H = torch.zeros(C, C, device=dev)
     ops.hessian_syrk_(H, X.to(dev), 0.0, 2.0 / n)
     H64 = O.hessian_fp64([X])
@@ -122,9 +125,10 @@ def test_hessian_syrk_vs_fp64(dev, n, C):
     assert torch.equal(Hc, Hc.t())  # mirrored exactly
 
 
-def test_hessian_running_mean_matches_oracle(dev):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_hessian_running_mean_matches_oracle(dev, dtype):
     C = 512
-    X = synth.activations_swiglu(3000, C, seed=9)
+    X = synth.activations_swiglu(3000, C, seed=9, dtype=dtype)
     chunks = [X[:700], X[700:701], X[701:2500], X[2500:]]
     H = torch.zeros(C, C, device=dev)
     Href, n = None, 0
@@ -137,12 +141,13 @@ def test_hessian_running_mean_matches_oracle(dev):
     assert ((H.cpu() - Href).norm() / Href.norm()).item() < 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("C,ns", [(512, [700, 300, 1500, 256, 4000]), (256, [300] * 18), (384, [100, 600, 0])])
-def test_hessian_syrk_grouped(dev, C, ns):
+def test_hessian_syrk_grouped(dev, C, ns, dtype):
     """Several Hessians in one call: each within the 1e-5 gate of fp64 and equal to the one-at-a-time result up to
     the order of the fp32 token sum."""
-    _say(f"grouped syrk C={C} ns={ns}")
-    Xs = [synth.activations_outlier(n, C, seed=50 + i) for i, n in enumerate(ns)]
+    _say(f"grouped syrk C={C} ns={ns} {dtype}")
+    Xs = [synth.activations_outlier(n, C, seed=50 + i, dtype=dtype) for i, n in enumerate(ns)]
     H0 = [_rand((C, C), 70 + i) for i in range(len(ns))]
     H0 = [h + h.t() for h in H0]
     betas = [0.25 * (i % 3) for i in range(len(ns))]

@@ -1,0 +1,165 @@
+"""Config 3, the whole-MoE-layer flow of quant.py:241-411 (all Hessians of the block first, then every linear
+quantized and packed; gate_proj and up_proj of an expert share one Hessian, quant.py:258-277):
+
+  (a) a reduced layer -- six experts at the real 2048x7168 / 7168x2048 shapes, skewed routing with one expert that
+      receives no token and one that receives fewer than 256 -- with EVERY linear compared with the CPU oracle fed
+      the oracle's own Hessian of that expert's routed tokens;
+  (b) the full layer (256 experts, 2,097,152 tokens, top-8) once, through checks that do not depend on size.
+"""
+import pytest
+import torch
+
+from moe_quant_amd import synth
+from moe_quant_amd.gptq import GPTQ
+from moe_quant_amd.moe_layer import ExpertWeights, quantize_moe_layer, route_tokens
+from oracle import gptq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(m):
+    print(m, flush=True)
+
+
+def _reduced_layer(dev, hidden=7168, inter=2048, tokens=6144, seed=31):
+    """Six experts; top-2 routing drawn from Zipf(1.1) weights over experts 0..3, expert 4 gets exactly 100 tokens,
+    expert 5 none."""
+    g = torch.Generator().manual_seed(seed)
+    x = synth.activations_outlier(tokens, hidden, seed)
+    p = 1.0 / torch.arange(1, 5).float() ** 1.1
+    ids = torch.stack([torch.multinomial(p, 2, replacement=False, generator=g) for _ in range(tokens)])
+    ids[:100, 1] = 4
+    experts = [ExpertWeights(synth.weight(inter, hidden, seed + 10 * e + 1).to(dev),
+                             synth.weight(inter, hidden, seed + 10 * e + 2).to(dev),
+                             synth.weight(hidden, inter, seed + 10 * e + 3).to(dev)) for e in range(6)]
+    return x, ids, experts
+
+
+def test_reduced_layer_every_linear_against_oracle(dev):
+    x, ids, experts = _reduced_layer(dev)
+    E = len(experts)
+    res = quantize_moe_layer(x.to(dev), ids.to(dev), experts, keep_outputs=True, keep_codes=list(range(E)), streams=3)
+    counts = torch.bincount(ids.flatten(), minlength=E).tolist()
+    _say(f"tokens per expert {counts}")
+    assert res.tokens_per_expert == counts and counts[4] == 100 and counts[5] == 0
+    rows, offsets = route_tokens(ids, E)
+    # expert 5 saw nothing: its three linears take the zero-sample fallback (round to nearest); nothing else is flagged
+    assert res.issues == {"zero_samples": 3, "nan_hessian": 0, "non_invertible": 0}
+    assert sorted(res.issues_by_linear) == ["5.down_proj", "5.gate_proj", "5.up_proj"]
+    # gate and up share one factorisation per expert, down has its own; the zero-sample expert still factors its
+    # identity matrices (as the reference does)
+    assert res.factorizations == 2 * E
+    for e in range(E):
+        xe = x[rows[offsets[e]:offsets[e + 1]]]
+        Hg = Hd = None
+        if xe.shape[0]:
+            Hg, n = O.hessian_update(None, 0, xe)
+            assert n == counts[e]
+            a = res.down_inputs[e].cpu()  # the expert forward is the model's part: the oracle gets the same activations
+            assert a.shape == (counts[e], experts[e].down.shape[1]) and a.dtype == torch.bfloat16
+            want = torch.nn.functional.silu(xe.float() @ experts[e].gate.cpu().float().t()) * (
+                xe.float() @ experts[e].up.cpu().float().t())
+            assert ((a.float() - want).norm() / want.norm()).item() < 1e-2  # bf16 forward
+            Hd, _ = O.hessian_update(None, 0, a)
+            for proj, Href in (("gate_proj", Hg), ("down_proj", Hd)):
+                got = res.hessians[f"{e}.{proj}"].cpu().double()
+                H64 = O.hessian_fp64([xe if proj == "gate_proj" else a])
+                assert ((got - H64).norm() / H64.norm()).item() < 1e-5, (e, proj)
+        for proj, W, Href in (("gate_proj", experts[e].gate, Hg), ("up_proj", experts[e].up, Hg),
+                              ("down_proj", experts[e].down, Hd)):
+            ref = O.quantize_linear(W.cpu(), None if Href is None else Href.clone())
+            q = res.qweight[f"{e}.{proj}"].cpu()
+            s = res.scales[f"{e}.{proj}"].cpu()
+            match = (q == ref["qweight"]).float().mean().item()
+            _say(f"  expert {e} {proj}: n={counts[e]} code match {match:.6f}")
+            assert torch.equal(s, ref["scale"]), (e, proj)
+            # a Hessian of rank 100 << C is held up by its damping term alone: rounding decisions sit closer together
+            assert match >= (0.999 if counts[e] != 100 else 0.995), (e, proj, match)
+            if Href is None:
+                assert torch.equal(q, ref["qweight"])  # round to nearest: exact
+            words = O.pack_weight({"qweight": q, "scale": s, "zero": torch.full_like(s, 8)}, 4, True, 128)["weight_packed"]
+            assert torch.equal(res.packed[f"{e}.{proj}"].cpu(), words), (e, proj)
+
+
+def test_layer_run_equals_one_linear_at_a_time(dev):
+    """The quantize phase of the layer driver (several linears in flight, shared factor for gate/up) against plain
+    GPTQ handles given the same Hessians and run one after another on one stream: bit-identical codes and scales."""
+    x, ids, experts = _reduced_layer(dev, hidden=1024, inter=512, tokens=4096, seed=77)
+    E = len(experts)
+    res = quantize_moe_layer(x.to(dev), ids.to(dev), experts, keep_codes=list(range(E)), streams=4)
+    for e in range(E):
+        for proj, W in (("gate_proj", experts[e].gate), ("up_proj", experts[e].up), ("down_proj", experts[e].down)):
+            lin = torch.nn.Linear(W.shape[1], W.shape[0], bias=False, dtype=W.dtype, device=dev)
+            lin.weight.data = W
+            h = GPTQ(lin, 128, True, 0.01, 128)
+            H = res.hessians.get(f"{e}.{proj.replace('up_proj', 'gate_proj')}")
+            if H is not None:
+                h.H, h.num_samples = H.clone(), res.tokens_per_expert[e]
+            q, s, z = h.quantize(4)
+            assert torch.equal(q, res.qweight[f"{e}.{proj}"]), (e, proj)
+            assert torch.equal(s, res.scales[f"{e}.{proj}"]), (e, proj)
+
+
+def test_full_layer_size_independent_properties(dev):
+    """256 experts x 3 linears, 2,097,152 tokens routed top-8 with Zipf-skewed loads, everything resident in HBM."""
+    n_exp, tokens = 256, 2_097_152
+    x, ids, ex = synth.moe_layer_on_device(dev, n_exp, tokens)
+    experts = [ExpertWeights(*w) for w in ex]
+    counts = torch.bincount(ids.flatten(), minlength=n_exp)
+    order = torch.argsort(counts, descending=True).tolist()
+    sample = [order[0], order[n_exp // 2], order[-1]]  # busiest, median, least loaded
+    _say(f"loads: max {int(counts.max())} median {int(counts.median())} min {int(counts.min())}; sample {sample}")
+    res = quantize_moe_layer(x, ids, experts, keep_outputs=True, keep_codes=sample)
+    _say(f"seconds {res.seconds}")
+    assert res.tokens_per_expert == counts.tolist() and sum(res.tokens_per_expert) == tokens * ids.shape[1]
+    assert res.issues == {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
+    assert res.factorizations == 2 * n_exp and len(res.packed) == 3 * n_exp
+    I, C = experts[0].gate.shape
+    for e in range(n_exp):  # every linear produced words and scales of the right shape and type
+        for proj, (R_, C_) in (("gate_proj", (I, C)), ("up_proj", (I, C)), ("down_proj", (C, I))):
+            w, s = res.packed[f"{e}.{proj}"], res.scales[f"{e}.{proj}"]
+            assert w.shape == (R_, C_ // 8) and w.dtype == torch.int32
+            assert s.shape == (R_, C_ // 128) and s.dtype == torch.bfloat16
+    rows, offsets = route_tokens(ids, n_exp)
+    for e in sample:
+        xe = x.index_select(0, rows[offsets[e]:offsets[e + 1]])
+        n = xe.shape[0]
+        inputs = {"gate_proj": xe, "up_proj": xe, "down_proj": res.down_inputs[e]}
+        for proj, W in (("gate_proj", experts[e].gate), ("up_proj", experts[e].up), ("down_proj", experts[e].down)):
+            key = f"{e}.{proj}"
+            q, s = res.qweight[key], res.scales[key]
+            # (1) the Hessian against torch's fp32 product of the same routed tokens
+            xin = inputs[proj]
+            Href = torch.zeros(xin.shape[1], xin.shape[1], device=dev)
+            for s0 in range(0, n, 32768):
+                blk = xin[s0:s0 + 32768].float()
+                Href.addmm_(blk.t(), blk)
+            Href.mul_(2.0 / n)
+            if proj != "up_proj":
+                assert ((res.hessians[key] - Href).norm() / Href.norm()).item() < 1e-5, key
+            # (2) scales equal the closed form; codes in range; words unpack to the codes
+            sg, _, _ = O.quantization_grid(W.cpu().float(), 128, 4, torch.bfloat16)
+            assert torch.equal(s.cpu(), sg.to(torch.bfloat16)), key
+            assert int(q.max()) <= 15
+            words = res.packed[key]
+            unpacked = torch.stack([(words >> (4 * i)) & 15 for i in range(8)], dim=-1).reshape(q.shape).to(torch.uint8)
+            assert torch.equal(unpacked, q), key
+            # (3) GPTQ beats round-to-nearest on the layer-output error tr(d H d^T)
+            Wf = W.float()
+            deq = (q.float() - 8.0) * s.float().repeat_interleave(128, dim=1)
+            srep = s.float().repeat_interleave(128, dim=1)
+            rtn = (torch.clamp(torch.floor(Wf / srep + 8.5), 0, 15) - 8.0) * srep
+            err = lambda d: ((d @ Href) * d).sum().item()
+            e_gptq, e_rtn = err(deq - Wf), err(rtn - Wf)
+            _say(f"  {key}: n={n} gptq/rtn output error {e_gptq / e_rtn:.3f}")
+            assert e_gptq < e_rtn, key
+            # (4) the same linear through a plain handle, alone on one stream: the same bits
+            lin = torch.nn.Linear(W.shape[1], W.shape[0], bias=False, dtype=W.dtype, device=dev)
+            lin.weight.data = W
+            h = GPTQ(lin, 128, True, 0.01, 128)
+            for s0 in range(0, n, 1 << 17):
+                h.update(xin[s0:s0 + (1 << 17)])
+            q1, s1, _ = h.quantize(4)
+            same = (q1 == q).float().mean().item()
+            _say(f"  {key}: stand-alone handle agrees on {same:.6f} of the codes")
+            assert torch.equal(s1, s) and same >= 0.999, key
