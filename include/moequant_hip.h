@@ -26,6 +26,7 @@ extern "C" {
 #define MQ_ERR_ARG (-1)
 #define MQ_ERR_LAUNCH (-2)
 #define MQ_ERR_WORKSPACE (-3)
+#define MQ_ERR_TOO_LARGE (-4)
 
 /* element types for `x_dtype` / `w_dtype` / `round_dtype` */
 #define MQ_DT_F32 0 /* round_dtype: no rounding */
@@ -98,6 +99,20 @@ int mq_hessian_prestep(float* H, long ldh, int C, int upper_only, uint8_t* prune
 size_t mq_hessian_damp_workspace_bytes(int C);
 int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_dtype, long ldw, int R, const uint8_t* pruned,
                     float rel_damp, int* flags, void* workspace, size_t workspace_bytes, void* stream);
+
+/* mq_hessian_damp without a workspace argument and without any allocation.  It has no counterpart in MoE-Quant: it
+ * exists for callers that cannot allocate or pass scratch memory -- code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  Same arguments, same kernels and bit-identical results; the scratch area
+ * (per-strip masks, dead-channel mask, damping scalar) is a device array inside the library, one copy per GPU, held
+ * until the process ends (17 * 32768 + 16 bytes, about 0.53 MiB).
+ *   Limit  : C <= 32768, otherwise MQ_ERR_TOO_LARGE and nothing is launched.
+ *   Sharing: every call on one GPU uses that GPU's one array: calls that overlap in time on one GPU (different
+ *            streams or host threads) race and must be serialised by the caller.  Nothing in the array needs to be
+ *            cleared between calls.
+ *   The first call on each device looks the array's address up (hipGetSymbolAddress); make that call outside
+ *   stream capture. */
+int mq_hessian_damp_noalloc(float* H, long ldh, int C, const void* W, int w_dtype, long ldw, int R,
+                            const uint8_t* pruned, float rel_damp, int* flags, void* stream);
 
 /* ---- (2) damped Cholesky / Cholesky-inverse -------------------------------------------------------
  * In place: A (SPD, upper triangle read, C % 128 == 0) -> unit-diagonal upper-triangular

@@ -8,7 +8,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmoequant_hip.so")
 
-MQ_OK, MQ_ERR_ARG, MQ_ERR_LAUNCH, MQ_ERR_WORKSPACE = 0, -1, -2, -3
+MQ_OK, MQ_ERR_ARG, MQ_ERR_LAUNCH, MQ_ERR_WORKSPACE, MQ_ERR_TOO_LARGE = 0, -1, -2, -3, -4
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 
 _vp, _i, _l, _f, _sz = C.c_void_p, C.c_int, C.c_long, C.c_float, C.c_size_t
@@ -25,6 +25,7 @@ SIGNATURES = {
     "mq_hessian_prestep": (_i, [_vp, _l, _i, _i, _vp, _vp, _vp]),
     "mq_hessian_damp_workspace_bytes": (_sz, [_i]),
     "mq_hessian_damp": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp, _sz, _vp]),
+    "mq_hessian_damp_noalloc": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp]),
     "mq_factor_upper_inverse": (_i, [_vp, _l, _i, _i, _vp, _vp]),
     "mq_factor_upper_inverse_from": (_i, [_vp, _l, _vp, _l, _i, _i, _vp, _vp]),
     "mq_quant_grid_sym": (_i, [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
@@ -64,7 +65,8 @@ def load():
     return lib
 
 
-_ERR = {MQ_ERR_ARG: "bad argument", MQ_ERR_LAUNCH: "kernel launch failed", MQ_ERR_WORKSPACE: "workspace too small"}
+_ERR = {MQ_ERR_ARG: "bad argument", MQ_ERR_LAUNCH: "kernel launch failed", MQ_ERR_WORKSPACE: "workspace too small",
+        MQ_ERR_TOO_LARGE: "problem larger than the entry point's fixed scratch capacity"}
 
 
 def check(rc: int, what: str) -> None:

@@ -7,6 +7,7 @@
 #define MQ_ERR_ARG (-1)       // bad pointer / size / alignment
 #define MQ_ERR_LAUNCH (-2)    // hipGetLastError() after a launch was not hipSuccess
 #define MQ_ERR_WORKSPACE (-3) // workspace too small
+#define MQ_ERR_TOO_LARGE (-4) // problem beyond the fixed capacity of an entry point that brings its own scratch memory
 // element types of weights, activations and rounding targets
 #define MQ_DT_F32 0
 #define MQ_DT_BF16 1

@@ -227,3 +227,41 @@ extern "C" int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_d
   hipLaunchKernelGGL(damp_apply_kernel, dim3(C), dim3(256), 0, st, H, ldh, C, dead, damp, flags);
   return mq_check_launch();
 }
+
+// ---------------------------------------------------------------------------------------------
+// mq_hessian_damp for callers that cannot hand over (or allocate) a workspace: code under HIP graph capture,
+// tight serving loops, harnesses that forbid allocation.  The strip masks, the dead-channel mask and the damping
+// scalar live in a device array that is part of the library image: every GPU the library runs on holds its own copy
+// (MQ_DAMP_NOALLOC_BYTES, about 0.53 MiB) until the process ends.
+// ---------------------------------------------------------------------------------------------
+namespace {
+constexpr int DAMP_NOALLOC_MAX_C = 32768;
+constexpr size_t DAMP_NOALLOC_BYTES = (size_t)(STRIPS + 1) * DAMP_NOALLOC_MAX_C + 16;
+constexpr int MAX_DEVICES = 64;
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[DAMP_NOALLOC_BYTES];
+
+extern "C" int mq_hessian_damp_noalloc(float* H, long ldh, int C, const void* W, int w_dtype, long ldw, int R,
+                                       const uint8_t* pruned, float rel_damp, int* flags, void* stream) {
+  if (C > DAMP_NOALLOC_MAX_C) return MQ_ERR_TOO_LARGE;
+  // `scratch` in host code is only a handle for the symbol: the array's device address is looked up once per
+  // device (each GPU has its own copy at its own address) and that pointer is what the kernels get.
+  static std::mutex mu;
+  static void* dev_ptr[MAX_DEVICES] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return MQ_ERR_LAUNCH;
+  void* ptr;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!dev_ptr[dev]) {
+      void* p = nullptr;
+      if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MQ_ERR_LAUNCH;
+      dev_ptr[dev] = p;
+    }
+    ptr = dev_ptr[dev];
+  }
+  // Nothing in the scratch area has to start at zero: the strip masks, the dead mask and the scalar are written in
+  // full by the first two kernels before the third reads them, so the previous call's contents do not matter.
+  return mq_hessian_damp(H, ldh, C, W, w_dtype, ldw, R, pruned, rel_damp, flags, ptr, DAMP_NOALLOC_BYTES, stream);
+}

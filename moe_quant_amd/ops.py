@@ -158,6 +158,22 @@ def hessian_damp_(H: Tensor, W: Tensor, pruned: Optional[Tensor], rel_damp: floa
     return H
 
 
+def hessian_damp_noalloc_(H: Tensor, W: Tensor, pruned: Optional[Tensor], rel_damp: float, flags: Tensor) -> Tensor:
+    """hessian_damp_ through the entry point that brings its own scratch memory: allocates nothing (neither here
+    nor in the library), C <= 32768, calls on one GPU must not overlap."""
+    _dev(H, W, pruned, flags)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    if W.dim() != 2 or W.shape[1] != C or W.stride(1) != 1:
+        raise ValueError("W must be (R,C) with unit column stride")
+    rc = lib.mq_hessian_damp_noalloc(H.data_ptr(), H.stride(0), C, W.data_ptr(), _dt(W.dtype), W.stride(0), W.shape[0],
+                                     _p(pruned), float(rel_damp), flags.data_ptr(), _stream(H))
+    check(rc, "mq_hessian_damp_noalloc")
+    return H
+
+
 # ---- (2) factorisation -------------------------------------------------------------------------------
 def factor_upper_inverse_(A: Tensor, info: Optional[Tensor] = None, normalize: bool = True) -> Tensor:
     """In place A -> upper U = chol(A^-1, upper), rows scaled to unit diagonal when `normalize`.
