@@ -28,8 +28,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--streams", type=int, default=4,
-                    help="independent linears are queued round-robin on this many HIP streams (1 = one at a time)")
+    ap.add_argument("--streams", type=int, default=2,
+                    help="groups of independent linears are queued round-robin on this many HIP streams")
+    ap.add_argument("--group", type=int, default=8,
+                    help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
     ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer"],
@@ -157,29 +159,36 @@ def main():
     layer.weight.data.copy_(case.W)
     X = case.X.to(dev)
 
-    def step():
-        h = GPTQ(layer, group_size=128, sym=True, rel_damp=0.01, block_size=128)
-        h.update(X)
-        q, s, z = h.quantize(4)
-        packed = h.packed_words()
-        return h, q, s, packed
+    def steps(g):
+        """g steps: g independent linears, each with its own Hessian, factor, codes and words."""
+        hs = [GPTQ(layer, group_size=128, sym=True, rel_damp=0.01, block_size=128) for _ in range(g)]
+        if g == 1:
+            hs[0].update(X)
+            outs = [hs[0].quantize(4)]
+        else:
+            GPTQ.update_many(hs, [X] * g)
+            outs = GPTQ.quantize_many(hs, 4)
+        packed = [h.packed_words() for h in hs]
+        return hs[-1], outs[-1][0], outs[-1][1], packed[-1]
 
-    # Steps are independent linears (each has its own Hessian, factor, codes and words).  One linear is a long
-    # chain of dependent launches that cannot fill the GPU by itself, so consecutive steps go round-robin
-    # onto `streams` HIP streams; nothing in a step reads a value back, the host just queues.
+    # Steps are independent linears.  One linear is a long chain of dependent launches that cannot fill the GPU by
+    # itself, so `group` consecutive steps share grouped library calls (every launch carries the work of all of
+    # them) and the groups go round-robin onto `streams` HIP streams; nothing in a step reads a value back, the
+    # host just queues.
     main_stream = torch.cuda.current_stream(dev)
     n_lanes = max(1, args.streams)
+    group = max(1, args.group)
     lanes = [main_stream] + [torch.cuda.Stream(device=dev) for _ in range(n_lanes - 1)]  # the current stream is lane 0
 
-    def run(k, lanes):
+    def run(k, lanes, group=group):
         for ln in lanes:
             if ln is not main_stream:
                 ln.wait_stream(main_stream)
         last = None
         t_begin = time.perf_counter()
-        for i in range(k):
-            with torch.cuda.stream(lanes[i % len(lanes)]):
-                last = step()
+        for bi, i in enumerate(range(0, k, group)):
+            with torch.cuda.stream(lanes[bi % len(lanes)]):
+                last = steps(min(group, k - i))
         host_ms[0] = (time.perf_counter() - t_begin) * 1e3 / max(k, 1)
         torch.cuda.synchronize()
         return last
@@ -191,9 +200,9 @@ def main():
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     host_issue_ms = host_ms[0]
     # the same step, one at a time on one stream: the latency of a single linear
-    run(1, [main_stream])
+    run(1, [main_stream], 1)
     t0 = time.perf_counter()
-    run(3, [main_stream])
+    run(3, [main_stream], 1)
     ms_single = (time.perf_counter() - t0) * 1e3 / 3
 
     # ---- per-phase device times (HIP events on the stream the kernels run on), outside the timed region
@@ -233,32 +242,25 @@ def main():
     codes = ops.untranspose_codes(Qt)
     t_pack_rc = timed(lambda: ops.pack_int4(codes), reps=10)
 
-    # the three big phases once more, `streams` independent calls in flight: device time per call when the chip is
-    # kept full (their sum is what a whole step costs at that many streams)
-    def per_call_in_flight(make_fn, reps=6):
-        fns = [make_fn(i) for i in range(len(lanes))]
-        for f in fns:
-            f()
-        torch.cuda.synchronize()
-        for ln in lanes:
-            if ln is not main_stream:
-                ln.wait_stream(main_stream)
-        t_begin = time.perf_counter()
-        for _ in range(reps):
-            for ln, f in zip(lanes, fns):
-                with torch.cuda.stream(ln):
-                    f()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t_begin) * 1e3 / (reps * len(lanes))
+    # the three big phases once more as the step runs them: one grouped library call over `group` linears on one
+    # stream; device time of the call / group
+    Gq = max(group, 1)
+    Hs = [torch.zeros(C, C, device=dev) for _ in range(Gq)]
+    t_syrk_g = timed(lambda: ops.hessian_syrk_grouped_(Hs, [X] * Gq, [0.0] * Gq, [2.0 / n] * Gq, mirror=False)) / Gq
+    del Hs
+    Hds = [Hd.clone() for _ in range(Gq)]
+    t_factor_g = timed(lambda: ops.factor_upper_inverse_from_grouped(Hds), reps=4) / Gq
+    del Hds
+    Wts = [torch.empty_like(Wt0) for _ in range(Gq)]
 
-    Hs = [torch.zeros(C, C, device=dev) for _ in lanes]
-    Wts = [torch.empty_like(Wt0) for _ in lanes]
-    infos = [torch.zeros(1, dtype=torch.int32, device=dev) for _ in lanes]
-    t_syrk_fl = per_call_in_flight(lambda i: (lambda: ops.hessian_syrk_(Hs[i], X, 0.0, 2.0 / n, mirror=False)))
-    t_factor_fl = per_call_in_flight(lambda i: (lambda: ops.factor_upper_inverse_from(Hd, infos[i])))
-    t_loop_fl = per_call_in_flight(lambda i: (lambda: (Wts[i].copy_(Wt0), ops.gptq_loop_(
-        Wts[i], A, s_gr, scale_row, None, 8.0, 15.0, torch.bfloat16, 128)))) - t_wcopy
-    del Hs, Wts
+    def loop_grouped():
+        for w in Wts:
+            w.copy_(Wt0)
+        ops.gptq_loop_grouped_(Wts, [A] * Gq, [s_gr] * Gq, [scale_row] * Gq, 8.0, 15.0, torch.bfloat16, 128)
+
+    t_loop_g = timed(loop_grouped) / Gq - t_wcopy
+    del Wts
+    torch.cuda.empty_cache()
 
     pts = torch.linspace(1, 0.2, 100, dtype=torch.float32, device=dev)
     s_try = s_rg.clone()
@@ -275,10 +277,13 @@ def main():
         "pack_from_loop_codes_ms": round(t_pack, 4),
         "pack_int4_ms": round(t_pack_rc, 4),
         "mse_scale_search_ms_not_in_step": round(t_mse, 4),
-        "streams_in_flight": len(lanes),
-        "hessian_syrk_ms_in_flight": round(t_syrk_fl, 4),
-        "factor_ms_in_flight": round(t_factor_fl, 4),
-        "gptq_loop_ms_in_flight": round(t_loop_fl, 4),
+        "linears_per_grouped_call": Gq,
+        "hessian_syrk_ms_per_linear_grouped": round(t_syrk_g, 4),
+        "factor_ms_per_linear_grouped": round(t_factor_g, 4),
+        "gptq_loop_ms_per_linear_grouped": round(t_loop_g, 4),
+        "hessian_syrk_frac_bf16_peak_grouped": round(flop_syrk / t_syrk_g / 1e9 / PEAK_BF16_MFMA, 4),
+        "factor_tflops_grouped": round(flop_factor / t_factor_g / 1e9, 2),
+        "gptq_loop_tflops_grouped": round(flop_loop / t_loop_g / 1e9, 2),
         "hessian_syrk_tflops": round(flop_syrk / t_syrk / 1e9, 2),
         "hessian_syrk_frac_bf16_peak": round(flop_syrk / t_syrk / 1e9 / PEAK_BF16_MFMA, 4),
         "factor_tflops": round(flop_factor / t_factor / 1e9, 2),
@@ -357,7 +362,7 @@ def main():
         "config": {
             "workload": "config 1: expert gate_proj 2048x7168 bf16, 8192 calibration tokens, 4-bit sym g128 B128; "
             "step = Hessian SYRK + factorisation + GPTQ loop + int32 packing",
-            "R": R, "C": C, "tokens": n, "streams": n_lanes,
+            "R": R, "C": C, "tokens": n, "streams": n_lanes, "linears_per_grouped_call": group,
         },
         "ms_per_step_one_stream": round(ms_single, 3),
         "host_queueing_ms_per_step": round(host_issue_ms, 3),

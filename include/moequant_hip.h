@@ -134,6 +134,32 @@ int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, 
 int mq_factor_upper_inverse_from(const float* H, long ldh, float* A, long lda, int C, int normalize, int* info,
                                  void* stream);
 
+/* `groups` matrices of one size C in one sequence of launches: the experts of an MoE block, which the reference
+ * factors one after another inside its per-linear loop (quant.py:291-386 calling src/gptq.py:236-242).  One
+ * factorisation is a chain of ~2 C/128 dependent launches with a one-workgroup step on its critical path and cannot
+ * fill the GPU; here every launch carries that step's work for all matrices, so the chain is paid once per call.
+ *   H, A, info : HOST arrays of `groups` device pointers (H[e] != A[e] for all e, or H[e] == A[e] for all e: in place);
+ *   ldh, lda, C, normalize : shared.  Results are bit-identical to `groups` separate calls.
+ *   Up to 16 matrices share a launch sequence; more run as consecutive batches. */
+int mq_factor_upper_inverse_grouped(int groups, const float* const* H, long ldh, float* const* A, long lda, int C,
+                                    int normalize, int* const* info, void* stream);
+
+/* Cholesky-only factorisation for the loop in its inverse-free form (mq_gptq_loop_chol).  Replaces the same torch calls
+ * as mq_factor_upper_inverse (src/linalg_utils.py:8-12, src/gptq.py:236-242) at half the flop: with H = R R^T, R upper,
+ * the factor of the inverse is U = R^-1, and the loop's recurrence  x_k = w_k + sum_{j<k} e_j U[j,k]/U[j,j]  (e_j the
+ * quantization error of column j, src/gptq_loop.py:141-148) is the same as
+ *     x_k = w_k - (1/R_kk) sum_{j<k} z_j R[j,k],    z_j = dequantized minus ORIGINAL weight of column j,
+ * so R^-1 is never needed.  Output: F[j,k] = -R[j,k] / R[k,k] for k > j; the diagonal and the lower triangle of F hold
+ * no defined values (the loop reads k > j only).  info and the identity fallback (F = 0 above the diagonal) as above.
+ *   H, F, info, workspace : as in mq_factor_upper_inverse_from; workspace = mq_factor_chol_workspace_bytes(C) bytes per
+ *   matrix (the 128x128 diagonal blocks of R), 16-byte aligned.  _grouped: HOST arrays of `groups` device pointers,
+ *   one launch sequence for up to 16 matrices at a time, results bit-identical to separate calls. */
+size_t mq_factor_chol_workspace_bytes(int C);
+int mq_factor_chol(const float* H, long ldh, float* F, long ldf, int C, int* info, void* workspace, size_t workspace_bytes,
+                   void* stream);
+int mq_factor_chol_grouped(int groups, const float* const* H, long ldh, float* const* F, long ldf, int C, int* const* info,
+                           void* const* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- (3) quantization grid and column loop ---------------------------------------------------------
  * Symmetric per-group scales.  Replaces find_quantization_meta (symmetric branch) as called from
  * get_quantization_grid, src/quant_utils.py:75-96,213-220:
@@ -163,6 +189,11 @@ int mq_mse_scale_sym(const void* W, int w_dtype, long ldw, int R, int C, int gro
 int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int* perm, const uint8_t* dead_cols,
                   float* Wt, long ldwt, void* stream);
 
+/* mq_prepare_wt writing the same values twice (Wt2 nullable): the inverse-free loop updates one copy in place and
+ * reads the original weights from the other. */
+int mq_prepare_wt_pair(const void* W, int w_dtype, long ldw, int R, int C, const int* perm, const uint8_t* dead_cols,
+                       float* Wt, float* Wt2, long ldwt, void* stream);
+
 /* The blocked GPTQ loop.  Replaces gptq_loop / gptq_loop_graph with both Triton kernels and the per-block
  * addmm_, src/gptq_loop.py:12-40,68-88,141-148.
  *   Wt    : C x R fp32 (ldw), in/out: original (permuted) weights in, dequantized weights out.
@@ -178,6 +209,29 @@ int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int*
 int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale, long ld_scale,
                  const int* scale_row, const float* qzero, float qzero_const, float maxq, int round_dtype, int block,
                  uint8_t* Qt, float* E, void* stream);
+
+/* The loop for `groups` linears of one shape (C, R, pitches, block, rounding and qzero_const shared) in one sequence
+ * of launches: every launch carries one block's column walk and trailing tiles for all of them (the reference runs
+ * its experts one after another, quant.py:291-386).  Wt, U, scale, scale_row, qzero, Qt, E: HOST arrays of `groups`
+ * device pointers, each as in mq_gptq_loop; scale_row / qzero may be NULL, otherwise their entries are all NULL or
+ * all set.  Every linear needs its own E ring.  Results are bit-identical to `groups` separate calls.
+ * Up to 16 linears share a launch sequence; more run as consecutive batches. */
+int mq_gptq_loop_grouped(int groups, float* const* Wt, long ldw, int C, int R, const float* const* U, long ldu,
+                         const float* const* scale, long ld_scale, const int* const* scale_row,
+                         const float* const* qzero, float qzero_const, float maxq, int round_dtype, int block,
+                         uint8_t* const* Qt, float* const* E, void* stream);
+
+/* The same loop (src/gptq_loop.py:12-40,68-88,141-148) in its inverse-free form: F from mq_factor_chol in U's place,
+ * and W0t, a read-only copy of the original Wt (mq_prepare_wt_pair), from which every column computes its total change
+ * z = y - w_original, the quantity handed on to later columns in place of the quantization error.  Same outputs as
+ * mq_gptq_loop on the corresponding U up to fp32 rounding; E holds z blocks.  _grouped as mq_gptq_loop_grouped. */
+int mq_gptq_loop_chol(float* Wt, const float* W0t, long ldw, int C, int R, const float* F, long ldf, const float* scale,
+                      long ld_scale, const int* scale_row, const float* qzero, float qzero_const, float maxq,
+                      int round_dtype, int block, uint8_t* Qt, float* E, void* stream);
+int mq_gptq_loop_chol_grouped(int groups, float* const* Wt, const float* const* W0t, long ldw, int C, int R,
+                              const float* const* F, long ldf, const float* const* scale, long ld_scale,
+                              const int* const* scale_row, const float* const* qzero, float qzero_const, float maxq,
+                              int round_dtype, int block, uint8_t* const* Qt, float* const* E, void* stream);
 
 /* codes[r, c] = Qt[perm_inv[c], r].  Replaces `[perm_inv].transpose(-2, -1).contiguous().to(torch.uint8)`,
  * src/gptq.py:199.  perm_inv nullable = identity. */

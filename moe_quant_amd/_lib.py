@@ -28,10 +28,18 @@ SIGNATURES = {
     "mq_hessian_damp_noalloc": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp]),
     "mq_factor_upper_inverse": (_i, [_vp, _l, _i, _i, _vp, _vp]),
     "mq_factor_upper_inverse_from": (_i, [_vp, _l, _vp, _l, _i, _i, _vp, _vp]),
+    "mq_factor_upper_inverse_grouped": (_i, [_i, _vp, _l, _vp, _l, _i, _i, _vp, _vp]),
+    "mq_factor_chol_workspace_bytes": (_sz, [_i]),
+    "mq_factor_chol": (_i, [_vp, _l, _vp, _l, _i, _vp, _vp, _sz, _vp]),
+    "mq_factor_chol_grouped": (_i, [_i, _vp, _l, _vp, _l, _i, _vp, _vp, _sz, _vp]),
     "mq_quant_grid_sym": (_i, [_vp, _i, _l, _i, _i, _i, _i, _vp, _i, _vp, _vp, _vp]),
     "mq_mse_scale_sym": (_i, [_vp, _i, _l, _i, _i, _i, _vp, _vp, _i, _f, _f, _f, _i, _vp, _vp, _vp]),
     "mq_prepare_wt": (_i, [_vp, _i, _l, _i, _i, _vp, _vp, _vp, _l, _vp]),
+    "mq_prepare_wt_pair": (_i, [_vp, _i, _l, _i, _i, _vp, _vp, _vp, _vp, _l, _vp]),
+    "mq_gptq_loop_chol": (_i, [_vp, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
+    "mq_gptq_loop_chol_grouped": (_i, [_i, _vp, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
     "mq_gptq_loop": (_i, [_vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
+    "mq_gptq_loop_grouped": (_i, [_i, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
     "mq_untranspose_codes": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
     "mq_pack_int4": (_i, [_vp, _l, _i, _i, _vp, _i, _vp, _l, _vp]),
     "mq_pack_from_qt": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),

@@ -86,7 +86,7 @@ def quantize_block(
 ) -> BlockReport:
     """`model`: any module whose linears under `prefix` are to be quantized (names as in `named_modules()`).
     `run_block()`: runs the block once over every calibration sequence (what quant.py:280-281 does); the forward
-    hooks installed here see the inputs of every linear.  Activations must be bf16."""
+    hooks installed here see the inputs of every linear (bf16, fp16 or fp32 activations)."""
     layers = select_layers(model, prefix, ".*", LINEAR_LAYERS)
     handles: Dict[str, GPTQ] = {}
     hooks = {}
@@ -156,7 +156,7 @@ def quantize_block(
                     if h.H is not None and lane is not main:
                         h.H.record_stream(lane)
                     h.H = None
-                    h._hessian_inv = None
+                    h._hessian_inv = h._loop_factor = None
                     h._Qt = None
                     h.W = h.layer.weight
         for ln in lanes:

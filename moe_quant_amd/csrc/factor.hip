@@ -180,8 +180,9 @@ __device__ __forceinline__ void tile_update(float* c, const float* a, const floa
 }
 //   tile_scale:  A(m,n) <- sum_{k >= n} A(m,k) * Xi(k,n), Xi = the lower-triangular Xt tile of the sub-block (in place)
 //   tr != nullptr: the result is final (an Xt tile of the inverse); its transpose is also stored at tr
+//   rd != nullptr: the result (a 32x32 piece of R) is also copied to global memory at rd (row pitch NB)
 template <bool COPY_T>
-__device__ __forceinline__ void tile_scale(float* a, const float* xi, float* tr, int lane) {
+__device__ __forceinline__ void tile_scale(float* a, const float* xi, float* tr, int lane, float* rd = nullptr) {
   int x = lane & 31;
   asm volatile("" : "+v"(x));  // keeps the masks below from being hoisted out of the caller's loops
   const int h = lane >> 5;
@@ -205,6 +206,7 @@ __device__ __forceinline__ void tile_scale(float* a, const float* xi, float* tr,
     t[2] = acc[4 * g + 2];
     t[3] = acc[4 * g + 3];
     *reinterpret_cast<floatx4*>(a + x * LDM + 8 * g + 4 * h) = t;
+    if (rd) *reinterpret_cast<floatx4*>(rd + x * NB + 8 * g + 4 * h) = t;
   }
   if (COPY_T) {
 #pragma unroll
@@ -216,7 +218,9 @@ constexpr int LDI = 36;  // row pitch of the 32x32 identity kept behind the matr
 
 // one wavefront: eliminate the diagonal sub-block at offset o; leaves the sub-block of the inverse in Xt and,
 // transposed, in the S triangle
-__device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, int gidx, int* info) {
+// rd != nullptr: rows of the 32x32 piece of R (valid from the diagonal on) are also copied to global memory at rd
+// (row pitch NB)
+__device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, int gidx, int* info, float* rd) {
   float reg[SB];
   const int li = lane & 31;
   const bool up = lane >= 32;
@@ -233,7 +237,14 @@ __device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, 
     reg[4 * q + 3] = t[3];
   }
   ElimStep<SB - 1>::run(reg, bcast_lane(reg[SB - 1], SB - 1), 0.f, 0.f, 0.f);
-  // The S rows are not written back: R itself is never read again.  The Xt rows hold the sub-block of the inverse.
+  if (rd && !up) {
+#pragma unroll
+    for (int q = 0; q < SB / 4; ++q) {
+      const floatx4 t = {reg[4 * q], reg[4 * q + 1], reg[4 * q + 2], reg[4 * q + 3]};
+      *reinterpret_cast<floatx4*>(rd + li * NB + 4 * q) = t;
+    }
+  }
+  // The S rows are not written back to LDS: R itself is never read again there.  The Xt rows hold the sub-block of the inverse.
   // First its transpose goes into the S triangle, where the finished inverse is collected row-major for the
   // write to memory (the zeros right of a row's diagonal land left of another row's: Xt or unused columns);
   // then the rows themselves, in place, for the products that follow (the quad that straddles the diagonal
@@ -257,8 +268,9 @@ __device__ __forceinline__ void eliminate_subblock(float* buf, int o, int lane, 
 // buf: LDS, NB*LDM floats followed by a 32 x LDI identity.  blk: global 128x128 block (row pitch ld).
 // gidx0: global index of its first row.  preloaded: the caller already filled Sv (upper) and zeroed the 32x32 Xt
 // tiles below the diagonal ones (a barrier here orders those writes).  blk rows must be 16-byte aligned.
+// rd (nullable): where the block R_bb of the factor itself goes, 128 x 128 row-major (valid on and above the diagonal).
 __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long ld, int gidx0, int* info,
-                                                  bool preloaded, const float* src = nullptr, long src_ld = 0) {
+                                                  bool preloaded, float* rd, const float* src = nullptr, long src_ld = 0) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int idx = tid; idx < SB * LDI; idx += 256) buf[NB * LDM + idx] = (idx / LDI == idx % LDI) ? 1.f : 0.f;
   if (preloaded) __syncthreads();
@@ -309,14 +321,14 @@ __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long l
       }
     }
     // ---- phase: elimination of the diagonal sub-block
-    if (wave == 0) eliminate_subblock(buf, o, lane, gidx0 + o, info);
+    if (wave == 0) eliminate_subblock(buf, o, lane, gidx0 + o, info, rd ? rd + o * NB + o : nullptr);
     __syncthreads();
     // ---- phase: column block J of M times the sub-block inverse: J row blocks of S above the diagonal,
     //      3-J row blocks of Xt below it (those are final: also copied, transposed, into the S triangle)
     for (int t = wave; t < 3; t += 4) {
       const bool is_s = t < J;
       const int ro = (is_s ? t : t + 1) * SB;
-      if (is_s) tile_scale<false>(buf + ro * LDM + o + SOFF, buf + o * LDM + o, nullptr, lane);
+      if (is_s) tile_scale<false>(buf + ro * LDM + o + SOFF, buf + o * LDM + o, nullptr, lane, rd ? rd + ro * NB + o : nullptr);
       else tile_scale<true>(buf + ro * LDM + o, buf + o * LDM + o, buf + o * LDM + ro + SOFF, lane);
     }
     __syncthreads();
@@ -335,11 +347,39 @@ __device__ __forceinline__ void diag_block_invert(float* buf, float* blk, long l
   }
 }
 
+// Several matrices of one size factored side by side: every launch carries the work of all of them.  The launch
+// sequence is written for matrix 0; a workgroup that serves matrix e shifts every pointer by the distance from
+// matrix 0's buffers to matrix e's (bytes: dA for the output buffers, dS for the input matrices).
+constexpr int MAX_GROUP = 16;
+struct FactorGroup {
+  long dA[MAX_GROUP], dS[MAX_GROUP], dW[MAX_GROUP];  // dW: the same for the workspaces of the Cholesky-only mode
+  int* info[MAX_GROUP];
+  int n;
+};
+template <typename P>
+__device__ __forceinline__ P* shifted(P* p, long bytes) {
+  return reinterpret_cast<P*>(reinterpret_cast<uintptr_t>(p) + bytes);
+}
+// smask: which pointers of g point into the input matrix (bit 0: A, 1: B, 2: C, 3: Csrc); the others point into the
+// output buffer
+__device__ __forceinline__ void rebase(GemmF32& g, const FactorGroup& grp, int e, int smask) {
+  const long dA = grp.dA[e], dS = grp.dS[e];
+  g.A = shifted(g.A, (smask & 1) ? dS : dA);
+  g.B = shifted(g.B, (smask & 2) ? dS : dA);
+  g.C = shifted(g.C, (smask & 4) ? dS : dA);
+  if (g.Csrc) g.Csrc = shifted(g.Csrc, (smask & 8) ? dS : dA);
+}
+
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void revchol_diag_kernel(const float* S, long lds,
                                                                                                     float* A, long ld, int i1,
-                                                                                                    int* info) {
+                                                                                                    FactorGroup grp, float* Rd) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, info, false, S + (long)i1 * lds + i1, lds);
+  const int e = blockIdx.x;
+  S = shifted(S, grp.dS[e]);
+  A = shifted(A, grp.dA[e]);
+  float* rd = Rd ? shifted(Rd, grp.dW[e]) + (long)i1 * NB : nullptr;  // block b = i1 / NB of the workspace
+  diag_block_invert(reinterpret_cast<float*>(smem), A + (long)i1 * ld + i1, ld, i1, grp.info[e], false, rd,
+                    S + (long)i1 * lds + i1, lds);
 }
 
 // The next diagonal tile, brought up to date by one workgroup on its own:  S(r,c) = H(r,c) - sum_k P(r,k) P(c,k)
@@ -434,8 +474,10 @@ __device__ __forceinline__ void inv_first_tile(const GemmF32& ginv, int kc, int 
   tile_body<false, true>(gl, tm, 0, 0, buf, 1, 1);
 }
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void inv_first_kernel(GemmF32 ginv, int kc) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void inv_first_kernel(GemmF32 ginv, int kc,
+                                                                                                 FactorGroup grp) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  rebase(ginv, grp, blockIdx.y, 0);
   inv_first_tile(ginv, kc, blockIdx.x, reinterpret_cast<float*>(smem));
 }
 
@@ -451,33 +493,51 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void i
 // The diagonal-block work is thereby hidden behind the bulk of the trailing update, and the inverse behind both.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void trail_diag_kernel(GemmF32 g, int total, GemmF32 ginv,
                                                                                                   int inv_tiles, int kc, float* A,
-                                                                                                  long ld, int i1, int* info,
-                                                                                                  int column_only) {
+                                                                                                  long ld, int i1, FactorGroup grp,
+                                                                                                  int column_only, int others,
+                                                                                                  int smask, float* Rd) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* buf = reinterpret_cast<float*>(smem);
   using namespace gemmf32;
-  const int bid = blockIdx.x;
+  // Workgroup order (a one-dimensional grid, so that what decides the launch's duration is dispatched first): the
+  // diagonal-block workgroups of all matrices, then the inverse tiles of all matrices, then the trailing tiles.
+  const int bid = blockIdx.x, G = grp.n;
+  int kind, e, idx;
+  if (bid < G) {
+    kind = 0, e = bid, idx = 0;
+  } else if (bid < G + G * inv_tiles) {
+    kind = 1, e = (bid - G) / inv_tiles, idx = (bid - G) % inv_tiles;
+  } else {
+    const int r = bid - G - G * inv_tiles;
+    kind = 2, e = r / others, idx = r % others;
+  }
+  e = __builtin_amdgcn_readfirstlane(e);
   // The workgroup on the dependence chain and the deep (K = 512) tiles of the inverse decide how long the launch
   // takes; each shares its CU with a stream of short K = 128 tiles.  Wave priority lets them have the matrix pipes
   // first: the short tiles lose what the long ones gain, the launch ends earlier.
-  if (bid <= inv_tiles) __builtin_amdgcn_s_setprio(3);
-  if (bid == 0) {
+  if (kind < 2) __builtin_amdgcn_s_setprio(3);
+  if (kind == 0) {
+    rebase(g, grp, e, smask);
+    A = shifted(A, grp.dA[e]);
     // (the last tile of the trailing update's upper-triangle order: the other workgroups cover total-1 tiles)
     // the whole tile goes to the S position: what lies left of a row's diagonal lands in that row's Xt or unused
     // columns, and the Xt part is cleared next
     diag_tile_update(buf, A, ld, i1, g.Csrc ? g.Csrc : A, g.Csrc ? g.ldcs : ld);
     __syncthreads();
     // Xt starts at zero in its 32x32 tiles below the diagonal ones (those are written whole by the elimination)
-    for (int idx = threadIdx.x; idx < (NB - SB) * (NB / 4); idx += 256) {
-      const int r = SB + idx / (NB / 4), q = idx % (NB / 4);
+    for (int idx2 = threadIdx.x; idx2 < (NB - SB) * (NB / 4); idx2 += 256) {
+      const int r = SB + idx2 / (NB / 4), q = idx2 % (NB / 4);
       if (q < (r / SB) * (SB / 4)) *reinterpret_cast<floatx4*>(buf + r * LDM + 4 * q) = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    diag_block_invert(buf, A + (long)(i1 - NB) * ld + (i1 - NB), ld, i1 - NB, info, true);
-  } else if (bid <= inv_tiles) {
-    inv_first_tile(ginv, kc, bid - 1, buf);
+    float* rd = Rd ? shifted(Rd, grp.dW[e]) + (long)(i1 - NB) * NB : nullptr;
+    diag_block_invert(buf, A + (long)(i1 - NB) * ld + (i1 - NB), ld, i1 - NB, grp.info[e], true, rd);
+  } else if (kind == 1) {
+    rebase(ginv, grp, e, 0);
+    inv_first_tile(ginv, kc, idx, buf);
   } else {
+    rebase(g, grp, e, smask);
     int tm, tn;
-    const int idx = bid - 1 - inv_tiles, T = i1 / NB;
+    const int T = i1 / NB;
     if (column_only) {  // block column T-1 above its diagonal tile, then the diagonal tile after that one
       tm = idx < T - 1 ? idx : T - 2;
       tn = idx < T - 1 ? T - 1 : T - 2;
@@ -491,13 +551,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void t
 // Panel product of step b (P = H_ab Dinv^T, 128 columns wide, in place: tiles of 64 rows x all 128 columns)
 // together with the second product of the inverse's block row b+1 (U12 = -U11 T, 128 rows high: tiles of
 // 64 x 64): two independent GEMMs with K = 128 in one launch.
-__global__ __launch_bounds__(256) void panel_inv_kernel(GemmF32 gp, int panel_tiles, GemmF32 g2, int inv_tiles) {
+__global__ __launch_bounds__(256) void panel_inv_kernel(GemmF32 gp, int panel_tiles, GemmF32 g2, int inv_tiles,
+                                                        FactorGroup grp, int smask_p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   float* buf = reinterpret_cast<float*>(smem);
-  const int bid = blockIdx.x;
+  const int bid = blockIdx.x, e = blockIdx.y;
   if (bid < panel_tiles) {
+    rebase(gp, grp, e, smask_p);
     gemmf32::tile_short<2>(gp, bid * 64, 0, buf);
   } else {
+    rebase(g2, grp, e, 0);
     const int r = bid - panel_tiles;
     gemmf32::tile_short<1>(g2, (r & 1) * 64, (r >> 1) * 64, buf);
   }
@@ -508,11 +571,11 @@ __global__ __launch_bounds__(256) void panel_inv_kernel(GemmF32 gp, int panel_ti
 // value before the barrier (a data dependence the compiler cannot reorder), so the thread that later
 // overwrites the diagonal cannot be observed by anyone.
 // A failed factorisation (*info != 0) leaves the identity, the fallback GPTQ takes when Cholesky raises.
-__global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C, int normalize, const int* info) {
+__global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C, int normalize, FactorGroup grp) {
   __shared__ float dsh;
   const int j = blockIdx.x;
-  float* row = A + (long)j * ld;
-  if (*info != 0) {
+  float* row = shifted(A, grp.dA[blockIdx.y]) + (long)j * ld;
+  if (*grp.info[blockIdx.y] != 0) {
     for (int k = threadIdx.x; k < C; k += 256) row[k] = (k == j) ? 1.f : 0.f;
     return;
   }
@@ -526,15 +589,76 @@ __global__ __launch_bounds__(256) void unit_diag_kernel(float* A, long ld, int C
   }
 }
 
+// Cholesky-only mode: the column loop can run on R itself (H = R R^T) instead of its inverse.  With z_j the total
+// change of column j (dequantized minus ORIGINAL weight), the value column k has when its turn comes is
+//   x_k = w_k - (1/R_kk) sum_{j<k} z_j R[j,k],
+// the same recurrence as the classical  x_k = w_k + sum_{j<k} e_j U[j,k]  (U = R^-1 with rows divided by the
+// diagonal, e_j the quantization error of column j): with y = x + e the classical form reads y = w + e D^-1 R^-1,
+// i.e. (y - w) R = e D^-1, which row k solves to the line above.  So the loop takes the multipliers
+//   F[j,k] = -R[j,k] / R[k,k]   (k > j)
+// and the triangular inverse, half the flop of the factorisation, is never formed.
+// One workgroup per upper 128x128 tile, in place: off-diagonal tiles hold R; a diagonal tile holds the inverse of
+// its block (of which only the diagonal, 1/R_kk, is used here), its R block comes from the workspace.  The diagonal
+// of F and everything below it is left as it is: the loop reads k > j only.
+// A failed factorisation (*info != 0) leaves F = 0 above the diagonal: the identity fallback of the reference.
+__global__ __launch_bounds__(256) void chol_finalize_kernel(float* A, long ld, int C, FactorGroup grp, const float* Rd) {
+  __shared__ float dcol[NB];
+  const int e = blockIdx.y;
+  A = shifted(A, grp.dA[e]);
+  Rd = shifted(Rd, grp.dW[e]);
+  int tm, tn;
+  gemmf32::tri_decode(blockIdx.x, tm, tn);
+  const int m0 = tm * NB, n0 = tn * NB, tid = threadIdx.x;
+  const bool failed = *grp.info[e] != 0;
+  if (tid < NB) dcol[tid] = A[(long)(n0 + tid) * ld + n0 + tid];  // 1 / R_kk
+  __syncthreads();
+#pragma unroll 4
+  for (int it = 0; it < 16; ++it) {
+    const int idx = tid + it * 256, r = idx >> 5, c = (idx & 31) << 2;
+    float* q = A + (long)(m0 + r) * ld + n0 + c;
+    if (tm != tn) {
+      floatx4 v = *reinterpret_cast<const floatx4*>(q);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = failed ? 0.f : -(v[i] * dcol[c + i]);
+      *reinterpret_cast<floatx4*>(q) = v;
+    } else if (c + 3 > r) {  // the quad holds at least one element right of the diagonal
+      const floatx4 rv = *reinterpret_cast<const floatx4*>(Rd + (long)(m0 + r) * NB + c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (c + i > r) q[i] = failed ? 0.f : -(rv[i] * dcol[c + i]);
+    }
+  }
+}
+
 constexpr size_t DIAG_SMEM = (size_t)(NB * LDM + SB * LDI) * sizeof(float);
 constexpr size_t FUSED_SMEM = DIAG_SMEM > gemmf32::SMEM_BYTES ? DIAG_SMEM : gemmf32::SMEM_BYTES;
 
 }  // namespace
 
-// S: the matrix to factor (upper triangle read), A: where the factor is built and left.  S == A: in place.
-static int factor_impl(const float* S, long lds, float* A, long ld, int C, int normalize, int* info, void* stream) {
-  if (!S || !A || !info || C <= 0 || ld < C || lds < C) return MQ_ERR_ARG;
+// S[e]: the matrices to factor (upper triangle read), A[e]: where the factors are built and left.  S[e] == A[e] for
+// every e: in place.  All matrices share C and the two pitches.
+// ws == nullptr: the inverse factor U.  ws[e] (C*128 floats each): Cholesky-only mode, the loop multipliers F.
+static int factor_impl(int G, const float* const* S, long lds, float* const* Aout, long ld, int C, int normalize,
+                       int* const* infos, float* const* ws, void* stream) {
+  if (G <= 0 || G > MAX_GROUP || !S || !Aout || !infos || C <= 0 || ld < C || lds < C) return MQ_ERR_ARG;
   if (C % NB != 0) return MQ_ERR_ARG;  // the host pads with an identity block
+  FactorGroup grp;
+  grp.n = G;
+  const bool in_place = S[0] == Aout[0];
+  for (int e = 0; e < MAX_GROUP; ++e) {
+    const int k = e < G ? e : 0;
+    if (!S[k] || !Aout[k] || !infos[k] || ((S[k] == Aout[k]) != in_place)) return MQ_ERR_ARG;
+    if ((ld & 3) || ((uintptr_t)Aout[k] & 15) || (lds & 3) || ((uintptr_t)S[k] & 15)) return MQ_ERR_ARG;  // float4 rows
+    grp.dA[e] = (long)((intptr_t)Aout[k] - (intptr_t)Aout[0]);
+    grp.dS[e] = (long)((intptr_t)S[k] - (intptr_t)S[0]);
+    grp.info[e] = infos[k];
+    if (ws && (!ws[k] || ((uintptr_t)ws[k] & 15))) return MQ_ERR_WORKSPACE;
+    grp.dW[e] = ws ? (long)((intptr_t)ws[k] - (intptr_t)ws[0]) : 0;
+  }
+  float* Rd = ws ? ws[0] : nullptr;
+  const bool chol = Rd != nullptr;
+  const float* S0 = S[0];
+  float* A = Aout[0];
   hipStream_t st = (hipStream_t)stream;
   static std::once_flag once;  // kernel attributes and tuning knobs: set once, whichever host thread comes first
   std::call_once(once, [] {
@@ -549,7 +673,6 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     (void)hipFuncSetAttribute((const void*)inv_first_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)gemmf32::SMEM_BYTES);
   });
-  if ((ld & 3) || ((uintptr_t)A & 15) || (lds & 3) || ((uintptr_t)S & 15)) return MQ_ERR_ARG;  // float4 access to rows
   int rc;
   auto kc_of = [&](int) { return INV_KC; };  // one depth for all block rows: 2, 3 for the short rows measured no faster
   // the two products of block row b of the inverse (w = columns to the right of b)
@@ -569,21 +692,21 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
                    NB, w, NB, -1.f, 0.f, 0, 0, 1, 0, 0, 0, (w / NB + kc_of(w) - 1) / kc_of(w), kc_of(w), NB};
   };
   const int B = C / NB;
-  hipLaunchKernelGGL(revchol_diag_kernel, dim3(1), dim3(256), DIAG_SMEM, st, S, lds, A, ld, C - NB, info);
+  hipLaunchKernelGGL(revchol_diag_kernel, dim3(G), dim3(256), DIAG_SMEM, st, S0, lds, A, ld, C - NB, grp, Rd);
   if ((rc = mq_check_launch()) != MQ_OK) return rc;
   for (int b = B - 1; b >= 1; --b) {
     const int i1 = b * NB;
     float* P = A + i1;  // panel: rows [0,i1), cols [i1, i1+NB)
     const float* Dinv = A + (long)i1 * ld + i1;
     // the first step reads what no earlier step has touched: from S (every later read finds its data in A)
-    const bool first = (b == B - 1) && (S != A);
-    GemmF32 panel{first ? S + i1 : P, Dinv, P, first ? lds : ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
+    const bool first = (b == B - 1) && !in_place;
+    GemmF32 panel{first ? S0 + i1 : P, Dinv, P, first ? lds : ld, 1, 1, ld, ld, i1, NB, NB, 1.f, 0.f, 0, 0, 1, 0, 0, 0};
     int t2 = 0;
     GemmF32 g2 = panel;
-    if (b + 1 <= B - 2) g2 = inv_second(b + 1, t2);  // row b+1: its T was produced in the previous launch
+    if (!chol && b + 1 <= B - 2) g2 = inv_second(b + 1, t2);  // row b+1: its T was produced in the previous launch
     static_assert(NB == gemmf32::SHORT_K, "the panel kernel's tiles take K = 128");
-    hipLaunchKernelGGL(panel_inv_kernel, dim3(2 * b + 4 * t2), dim3(256), gemmf32::short_smem_bytes(2), st, panel, 2 * b,
-                       g2, 4 * t2);
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(2 * b + 4 * t2, G), dim3(256), gemmf32::short_smem_bytes(2), st, panel, 2 * b,
+                       g2, 4 * t2, grp, first ? 1 : 0);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     // The trailing update A[0:i1,0:i1] -= P P^T with one 128-wide panel is bound by reading and writing the
     // trailing matrix, so after the first step (which also carries the matrix from S to A) the panels go in
@@ -600,44 +723,85 @@ static int factor_impl(const float* S, long lds, float* A, long ld, int C, int n
     const int column_only = step >= 1 && j < TRAIL_PANELS;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, j * NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     if (first) {
-      trail.Csrc = S;
+      trail.Csrc = S0;
       trail.ldcs = lds;
     }
     const int tiles = i1 / NB, total = tiles * (tiles + 1) / 2;
     const int others = column_only ? (b - 1) + (b >= 2 ? 1 : 0) : total - 1;  // tiles besides workgroup 0's
     int t1 = 0;
     GemmF32 g1 = trail;
-    if (b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
-    hipLaunchKernelGGL(trail_diag_kernel, dim3(1 + t1 + others), dim3(256), FUSED_SMEM, st, trail, total, g1, t1,
-                       kc_of(C - i1 - NB), A, ld, i1, info, column_only);
+    if (!chol && b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
+    hipLaunchKernelGGL(trail_diag_kernel, dim3(G * (1 + t1 + others)), dim3(256), FUSED_SMEM, st, trail, total, g1, t1,
+                       kc_of(C - i1 - NB), A, ld, i1, grp, column_only, others, first ? 8 : 0, Rd);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
+  }
+  if (chol) {
+    hipLaunchKernelGGL(chol_finalize_kernel, dim3(B * (B + 1) / 2, G), dim3(256), 0, st, A, ld, C, grp, (const float*)Rd);
+    return mq_check_launch();
   }
   // what is left of the inverse once the elimination has reached the top: second product of row 1, both of row 0
   if (B >= 3) {
     int t2;
     GemmF32 g2 = inv_second(1, t2);
-    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t2), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t2);
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t2, G), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t2, grp,
+                       0);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
   if (B >= 2) {
     int t;
     GemmF32 g1 = inv_first(0, t);
-    hipLaunchKernelGGL(inv_first_kernel, dim3(t), dim3(256), gemmf32::SMEM_BYTES, st, g1, kc_of(C - NB));
+    hipLaunchKernelGGL(inv_first_kernel, dim3(t, G), dim3(256), gemmf32::SMEM_BYTES, st, g1, kc_of(C - NB), grp);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
     GemmF32 g2 = inv_second(0, t);
-    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t);
+    hipLaunchKernelGGL(panel_inv_kernel, dim3(4 * t, G), dim3(256), gemmf32::short_smem_bytes(2), st, g2, 0, g2, 4 * t, grp,
+                       0);
     if ((rc = mq_check_launch()) != MQ_OK) return rc;
   }
-  hipLaunchKernelGGL(unit_diag_kernel, dim3(C), dim3(256), 0, st, A, ld, C, normalize, info);
+  hipLaunchKernelGGL(unit_diag_kernel, dim3(C, G), dim3(256), 0, st, A, ld, C, normalize, grp);
   return mq_check_launch();
 }
 
 extern "C" int mq_factor_upper_inverse(float* A, long ld, int C, int normalize, int* info, void* stream) {
-  return factor_impl(A, ld, A, ld, C, normalize, info, stream);
+  const float* S = A;
+  return factor_impl(1, &S, ld, &A, ld, C, normalize, &info, nullptr, stream);
 }
 
 extern "C" int mq_factor_upper_inverse_from(const float* H, long ldh, float* A, long lda, int C, int normalize, int* info,
                                             void* stream) {
   if (H == A) return MQ_ERR_ARG;
-  return factor_impl(H, ldh, A, lda, C, normalize, info, stream);
+  return factor_impl(1, &H, ldh, &A, lda, C, normalize, &info, nullptr, stream);
+}
+
+// `groups` matrices of one size in one sequence of launches (host arrays of device pointers).  More than MAX_GROUP
+// matrices run as consecutive batches.
+extern "C" int mq_factor_upper_inverse_grouped(int groups, const float* const* H, long ldh, float* const* A, long lda, int C,
+                                               int normalize, int* const* info, void* stream) {
+  if (groups < 0 || (groups > 0 && (!H || !A || !info))) return MQ_ERR_ARG;
+  for (int g0 = 0; g0 < groups; g0 += MAX_GROUP) {
+    const int cnt = groups - g0 < MAX_GROUP ? groups - g0 : MAX_GROUP;
+    const int rc = factor_impl(cnt, H + g0, ldh, A + g0, lda, C, normalize, info + g0, nullptr, stream);
+    if (rc != MQ_OK) return rc;
+  }
+  return MQ_OK;
+}
+
+// Cholesky-only mode (see chol_finalize_kernel): F[j,k] = -R[j,k] / R[k,k] for k > j, H = R R^T, in F's upper
+// triangle; the diagonal and the lower triangle of F hold no defined values.
+extern "C" size_t mq_factor_chol_workspace_bytes(int C) { return C > 0 ? (size_t)C * NB * sizeof(float) : 0; }
+
+extern "C" int mq_factor_chol_grouped(int groups, const float* const* H, long ldh, float* const* F, long ldf, int C,
+                                      int* const* info, void* const* workspace, size_t workspace_bytes, void* stream) {
+  if (groups < 0 || (groups > 0 && (!H || !F || !info || !workspace))) return MQ_ERR_ARG;
+  if (workspace_bytes < mq_factor_chol_workspace_bytes(C)) return MQ_ERR_WORKSPACE;
+  for (int g0 = 0; g0 < groups; g0 += MAX_GROUP) {
+    const int cnt = groups - g0 < MAX_GROUP ? groups - g0 : MAX_GROUP;
+    const int rc = factor_impl(cnt, H + g0, ldh, F + g0, ldf, C, 1, info + g0, (float* const*)(workspace + g0), stream);
+    if (rc != MQ_OK) return rc;
+  }
+  return MQ_OK;
+}
+
+extern "C" int mq_factor_chol(const float* H, long ldh, float* F, long ldf, int C, int* info, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  return mq_factor_chol_grouped(1, &H, ldh, &F, ldf, C, &info, &workspace, workspace_bytes, stream);
 }

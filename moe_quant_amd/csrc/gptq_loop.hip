@@ -17,6 +17,11 @@
 //
 // Arithmetic per column is the reference's: q = clamp(floor(x/s + z + 0.5), 0, maxq) with IEEE division,
 // y = round_to(dtype)((q - z) * s), e = y - x, w_k = fma(U[j,k], e, w_k).
+//
+// Second mode (ZMODE, mq_gptq_loop_chol): the same recurrence written on the Cholesky factor of H itself instead of
+// the factor of its inverse (see mq_factor_chol): the multipliers are F[j,k] = -R[j,k]/R[k,k] and what a column hands
+// on is not its quantization error but its total change z = y - w_original.  Nothing else differs: same walk, same
+// lazy batches; the original weights come from a second, read-only copy of the transposed weights.
 #include <hip/hip_fp16.h>
 
 #include <cstdlib>
@@ -37,6 +42,26 @@ __device__ __forceinline__ float round_dtype(float x, int rd) {
   const float h = __half2float(__float2half_rn(x));
   return rd == 1 ? b : (rd == 2 ? h : x);
 }
+
+// Several linears of one shape walked side by side: every launch carries the column workgroups and the trailing
+// tiles of all of them.  Per linear its own buffers; everything else (sizes, pitches, block schedule) is shared.
+constexpr int MAX_GROUP = 16;
+struct LoopGroup {
+  float* Wt[MAX_GROUP];
+  const float* U[MAX_GROUP];
+  const float* scale[MAX_GROUP];
+  const int* scale_row[MAX_GROUP];
+  const float* qzero[MAX_GROUP];
+  uint8_t* Qt[MAX_GROUP];
+  float* E[MAX_GROUP];
+  const float* W0t[MAX_GROUP];  // ZMODE: the original weights, laid out like Wt
+  int n;
+};
+// where this launch's pieces lie inside a linear's buffers (elements)
+struct LoopOffsets {
+  long e_cur, e_prev;       // error block written / folded in by the column workgroups (e_prev < 0: none)
+  long g_a, g_b, g_c;       // trailing update: A inside U, B inside E, C inside Wt
+};
 
 struct LoopArgs {
   float* Wt;
@@ -140,10 +165,10 @@ struct WalkFma {  // w[T..15] += U[j, T..] * e
   }
 };
 
-template <bool FULL, int RD, bool RCP, int J>
+template <bool FULL, int RD, bool RCP, bool ZMODE, int J>
 struct WalkStep {
   static __device__ __forceinline__ void run(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB],
-                                             const float (&u)[MB], const WalkCtx& c) {
+                                             const float (&u)[MB], const float (&w0)[MB], const WalkCtx& c) {
     if constexpr (J < MB) {
       const float s = sc[J], z = zz[J];
       const float x = w[J];
@@ -165,7 +190,7 @@ struct WalkStep {
       } else if (RD == 2) {
         y = __half2float(__float2half_rn(d));
       }
-      const float e = (FULL || J < c.left) ? (y - x) : 0.f;
+      const float e = (FULL || J < c.left) ? (y - (ZMODE ? w0[J] : x)) : 0.f;
       WalkFma<J + 1, J>::run(w, u[J], e);  // the next column first: it is the dependence chain
       c.esh_lane[J * WSTRIDE] = e;
       if (FULL || J < c.left) {
@@ -174,18 +199,18 @@ struct WalkStep {
         c.eout[(long)J * c.R] = e;
       }
       __builtin_amdgcn_sched_barrier(0);
-      WalkStep<FULL, RD, RCP, J + 1>::run(w, sc, zz, u, c);
+      WalkStep<FULL, RD, RCP, ZMODE, J + 1>::run(w, sc, zz, u, w0, c);
     }
   }
 };
 
-template <bool FULL, int RD, bool RCP>
+template <bool FULL, int RD, bool RCP, bool ZMODE>
 __device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], const float (&zz)[MB], const float* ut,
-                                       int c0, int lane, const WalkCtx& c) {
+                                       int c0, int lane, const float (&w0)[MB], const WalkCtx& c) {
   float u[MB];  // row J of the micro-block of U: lane l holds U[c0+J, c0 + l%16]
 #pragma unroll
   for (int J = 0; J < MB; ++J) u[J] = ut[ut_off(c0 + J, c0) + (lane & 15)];
-  WalkStep<FULL, RD, RCP, 0>::run(w, sc, zz, u, c);
+  WalkStep<FULL, RD, RCP, ZMODE, 0>::run(w, sc, zz, u, w0, c);
 }
 
 // One workgroup (four wavefronts) owns 64 rows; lane l of every wavefront is row l.  The 128-column
@@ -200,21 +225,37 @@ __device__ __forceinline__ void walk16(float (&w)[MB], const float (&sc)[MB], co
 // Nothing else runs on the CU to hide latency, so every phase issues its loads in bulk before the first
 // use: the kernel is built from branch-free unrolled blocks for that reason (ROWMAP / QZERO are template
 // flags, the rounding mode is a select).
-template <bool FULL, bool ROWMAP, bool QZERO>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gptq_block_kernel(LoopArgs a, int i1, int nb, int col_wgs, GemmF32 g, int tiles_n,
-                                                        int vecA, int vecB) {
+template <bool FULL, bool ROWMAP, bool QZERO, bool ZMODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gptq_block_kernel(LoopArgs a, int i1, int nb, int col_wgs, GemmF32 g, int tiles,
+                                                        int tiles_n, int vecA, int vecB, LoopGroup grp, LoopOffsets off) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  if ((int)blockIdx.x >= col_wgs) {  // a tile of the previous block's trailing update
-    const int idx = blockIdx.x - col_wgs;
+  // workgroup order: the column workgroups of every linear first (they decide how long the launch takes), then
+  // the trailing tiles
+  const int bid = blockIdx.x, ncol = grp.n * col_wgs;
+  const int e = __builtin_amdgcn_readfirstlane(bid < ncol ? bid / col_wgs : (bid - ncol) / tiles);
+  a.Wt = grp.Wt[e];
+  a.U = grp.U[e];
+  a.scale = grp.scale[e];
+  a.scale_row = grp.scale_row[e];
+  a.qzero = grp.qzero[e];
+  a.Qt = grp.Qt[e];
+  a.E = grp.E[e] + off.e_cur;
+  a.Eprev = off.e_prev >= 0 ? grp.E[e] + off.e_prev : nullptr;
+  if (bid >= ncol) {  // a tile of the trailing update due at this block
+    const int idx = (bid - ncol) % tiles;
+    g.A = a.U + off.g_a;
+    g.B = grp.E[e] + off.g_b;
+    g.C = a.Wt + off.g_c;
     gemmf32::tile_body<false, false>(g, idx / tiles_n, idx % tiles_n, 0, reinterpret_cast<float*>(smem), vecA, vecB);
     return;
   }
+  const int wg = bid % col_wgs;
   float* tile = reinterpret_cast<float*>(smem);  // [B][WSTRIDE]
   float* ut = tile + B * WSTRIDE;                // packed upper micro-blocks of the U block
   float* esh = ut + UT_FLOATS;                   // [2][MB][WSTRIDE] errors of the current and the previous micro-block
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: row addresses below stay in scalar registers
-  const int r0 = blockIdx.x * 64;
+  const int r0 = wg * 64;
   // Lanes past the last row shadow row R-1: they compute and store exactly what that row's own lane
   // does, so no branch in this kernel ever diverges.
   const int r = min(r0 + lane, a.R - 1);
@@ -346,12 +387,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
       rcp_blk = 1.0f / sc_blk;
     }
   }
+  // ZMODE: the original weights of the micro-block about to be walked, fetched one micro-block ahead by wavefront 0
+  // (the walk of a micro-block hides the round trip)
+  float w0n[MB];
+  const float* w0p = ZMODE ? grp.W0t[e] + (long)i1 * a.ldw + r : nullptr;
+  if (ZMODE && wave == 0) {
+#pragma unroll
+    for (int t = 0; t < MB; ++t) w0n[t] = w0p[(long)min(t, nb - 1) * a.ldw];
+  }
 #pragma unroll 1
   for (int c0 = 0; c0 < cend; c0 += MB) {
     const float* eprev = esh + (((c0 / MB) + 1) & 1) * MB * WSTRIDE;
     float* ecur = esh + ((c0 / MB) & 1) * MB * WSTRIDE;
     if (wave == 0) {
-      float w[MB], sc[MB], zz[MB];
+      float w[MB], sc[MB], zz[MB], w0[MB];
+      if (ZMODE) {
+#pragma unroll
+        for (int t = 0; t < MB; ++t) w0[t] = w0n[t];
+#pragma unroll
+        for (int t = 0; t < MB; ++t) w0n[t] = w0p[(long)min(c0 + MB + t, nb - 1) * a.ldw];
+      } else {
+#pragma unroll
+        for (int t = 0; t < MB; ++t) w0[t] = 0.f;
+      }
       if (one_row) {
 #pragma unroll
         for (int t = 0; t < MB; ++t) {
@@ -372,7 +430,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
       const float* utd = ut;
       const WalkCtx wc{rcp_blk, maxq, nb - c0, ecur + lane, wp + (long)c0 * a.ldw, a.ldw,
                        a.Qt + (long)(i1 + c0) * a.R + r, a.E + (long)c0 * a.R + r, a.R};
-#define MQ_WALK(RD_, RCP_) walk16<FULL, RD_, RCP_>(w, sc, zz, utd, c0, lane, wc)
+#define MQ_WALK(RD_, RCP_) walk16<FULL, RD_, RCP_, ZMODE>(w, sc, zz, utd, c0, lane, w0, wc)
       if (one_row) {
         if (rd == 1) MQ_WALK(1, true);
         else if (rd == 2) MQ_WALK(2, true);
@@ -432,14 +490,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 constexpr size_t COL_SMEM = (size_t)(B * WSTRIDE + UT_FLOATS + 2 * MB * WSTRIDE) * sizeof(float);
 constexpr size_t BLOCK_SMEM = COL_SMEM > gemmf32::SMEM_BYTES ? COL_SMEM : gemmf32::SMEM_BYTES;
 
-template <bool ROWMAP, bool QZERO>
-int run_loop(const LoopArgs& a, int block, hipStream_t st) {
-  const int grid = (a.R + 63) / 64;
+template <bool ROWMAP, bool QZERO, bool ZMODE>
+int run_loop(const LoopArgs& a, const LoopGroup& grp, int block, hipStream_t st) {
+  const int grid = (a.R + 63) / 64, G = grp.n;
   static std::once_flag once;  // one per template instance
   std::call_once(once, [] {
-    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<true, ROWMAP, QZERO>,
+    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<true, ROWMAP, QZERO, ZMODE>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
-    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO>,
+    (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO, ZMODE>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
     if (const char* e = getenv("MQ_LOOP_BATCH")) {
       const int v = atoi(e);
@@ -454,8 +512,9 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
     // Error blocks live in a ring of 2 * LOOP_BATCH: this block's, the previous one (the column workgroups fold it
     // into their own columns) and the batches a trailing update may still be reading.
     const int RING = 2 * LOOP_BATCH;  // a multiple of the batch: an aligned batch never wraps
-    la.E = a.E + (long)(blk % RING) * B * a.R;
-    la.Eprev = blk ? a.E + (long)((blk - 1) % RING) * B * a.R : nullptr;
+    LoopOffsets off;
+    off.e_cur = (long)(blk % RING) * B * a.R;
+    off.e_prev = blk ? (long)((blk - 1) % RING) * B * a.R : -1;
     la.nbprev = nbprev;
     // Trailing updates, Wt[i2+m, r] += sum_j U[j0+j, i2+m] * E[j, r], run beside the column walk of this block.
     // A rank-128 update of everything beyond is bound by reading and writing those columns, so with 128-column
@@ -464,31 +523,37 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
     // blk >= D: the batch just completed into everything beyond (K = 128 D); otherwise the r errors of the batch
     // under way into the next block only (K = 128 r).
     // Other block widths: the previous block's errors into everything beyond, every time.
-    GemmF32 g{a.U, la.Eprev, a.Wt + (long)i2 * a.ldw, 1, a.ldu, a.R, 1, a.ldw, a.C - i2, a.R, nbprev, 1.f, 1.f,
-              0, 0, 1, 0, 0, 0};
+    // (the pointers of g are filled in by the kernel from the offsets: they differ from linear to linear)
+    GemmF32 g{nullptr, nullptr, nullptr, 1, a.ldu, a.R, 1, a.ldw, a.C - i2, a.R, nbprev, 1.f, 1.f, 0, 0, 1, 0, 0, 0};
+    off.g_a = off.g_b = off.g_c = 0;
     int tiles = 0, tiles_n = 1, vecA = 0, vecB = 0;
     if (blk && i2 < a.C) {
       long j0 = i1 - nbprev;
+      off.g_b = off.e_prev;
       if (block == B) {
         const int D = LOOP_BATCH, r = blk % D;
         const int first = r ? blk - r : blk - D;  // first block of the errors applied now
         if (r) g.M = (a.C - i2 < block) ? a.C - i2 : block;
         j0 = (long)first * B;
-        g.B = a.E + (long)(first % RING) * B * a.R;
+        off.g_b = (long)(first % RING) * B * a.R;
         g.K = (blk - first) * B;
       }
-      g.A = a.U + j0 * a.ldu + i2;
+      off.g_a = j0 * a.ldu + i2;
+      off.g_c = (long)i2 * a.ldw;
       tiles_n = (a.R + gemmf32::BN - 1) / gemmf32::BN;
       tiles = ((g.M + gemmf32::BM - 1) / gemmf32::BM) * tiles_n;
-      vecA = mq_gemm_operand_aligned(g.A, g.sak, 0);
-      vecB = mq_gemm_operand_aligned(g.B, g.sbk, 0);
+      vecA = vecB = 1;
+      for (int e = 0; e < G; ++e) {
+        vecA &= (int)mq_gemm_operand_aligned(grp.U[e] + off.g_a, g.sak, 0);
+        vecB &= (int)mq_gemm_operand_aligned(grp.E[e] + off.g_b, g.sbk, 0);
+      }
     }
     if (nb == B)
-      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO>), dim3(grid + tiles), dim3(256), BLOCK_SMEM, st, la, i1,
-                         nb, grid, g, tiles_n, vecA, vecB);
+      hipLaunchKernelGGL((gptq_block_kernel<true, ROWMAP, QZERO, ZMODE>), dim3(G * (grid + tiles)), dim3(256), BLOCK_SMEM, st, la,
+                         i1, nb, grid, g, tiles, tiles_n, vecA, vecB, grp, off);
     else
-      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO>), dim3(grid + tiles), dim3(256), BLOCK_SMEM, st, la, i1,
-                         nb, grid, g, tiles_n, vecA, vecB);
+      hipLaunchKernelGGL((gptq_block_kernel<false, ROWMAP, QZERO, ZMODE>), dim3(G * (grid + tiles)), dim3(256), BLOCK_SMEM, st, la,
+                         i1, nb, grid, g, tiles, tiles_n, vecA, vecB, grp, off);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
     nbprev = nb;
@@ -496,17 +561,91 @@ int run_loop(const LoopArgs& a, int block, hipStream_t st) {
   return MQ_OK;
 }
 
+// W0t == nullptr: the classical loop on U.  W0t[e] (original weights, laid out like Wt[e]): the loop on the Cholesky
+// multipliers F, passed in U's place.
+int loop_impl(int G, float* const* Wt, long ldw, int C, int R, const float* const* U, long ldu, const float* const* scale,
+              long ld_scale, const int* const* scale_row, const float* const* qzero, float qzero_const, float maxq,
+              int round_dtype, int block, uint8_t* const* Qt, float* const* E, const float* const* W0t, void* stream) {
+  if (G <= 0 || G > MAX_GROUP || !Wt || !U || !scale || !Qt || !E || C <= 0 || R <= 0) return MQ_ERR_ARG;
+  if (ldw < R || ldu < C || ld_scale < R) return MQ_ERR_ARG;
+  if (round_dtype < 0 || round_dtype > 2) return MQ_ERR_ARG;
+  if (block <= 0 || block > B) block = B;  // wider blocks only reassociate the trailing sums
+  LoopGroup grp;
+  grp.n = G;
+  const bool rowmap = scale_row && scale_row[0], qz = qzero && qzero[0];
+  for (int e = 0; e < MAX_GROUP; ++e) {
+    const int k = e < G ? e : 0;
+    if (!Wt[k] || !U[k] || !scale[k] || !Qt[k] || !E[k]) return MQ_ERR_ARG;
+    if (((scale_row && scale_row[k]) != rowmap) || ((qzero && qzero[k]) != qz)) return MQ_ERR_ARG;  // all or none
+    grp.Wt[e] = Wt[k];
+    grp.U[e] = U[k];
+    grp.scale[e] = scale[k];
+    grp.scale_row[e] = rowmap ? scale_row[k] : nullptr;
+    grp.qzero[e] = qz ? qzero[k] : nullptr;
+    grp.Qt[e] = Qt[k];
+    grp.E[e] = E[k];
+    if (W0t && (!W0t[k] || W0t[k] == Wt[k])) return MQ_ERR_ARG;
+    grp.W0t[e] = W0t ? W0t[k] : nullptr;
+  }
+  LoopArgs a{Wt[0], ldw, C, R, U[0], ldu, scale[0], ld_scale, grp.scale_row[0], grp.qzero[0], qzero_const, maxq,
+             round_dtype, Qt[0], E[0], nullptr, 0};
+  hipStream_t st = (hipStream_t)stream;
+  if (W0t) {
+    if (rowmap) return qz ? run_loop<true, true, true>(a, grp, block, st) : run_loop<true, false, true>(a, grp, block, st);
+    return qz ? run_loop<false, true, true>(a, grp, block, st) : run_loop<false, false, true>(a, grp, block, st);
+  }
+  if (rowmap) return qz ? run_loop<true, true, false>(a, grp, block, st) : run_loop<true, false, false>(a, grp, block, st);
+  return qz ? run_loop<false, true, false>(a, grp, block, st) : run_loop<false, false, false>(a, grp, block, st);
+}
+
 }  // namespace
 
 extern "C" int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale,
                             long ld_scale, const int* scale_row, const float* qzero, float qzero_const, float maxq,
                             int round_dtype, int block, uint8_t* Qt, float* E, void* stream) {
-  if (!Wt || !U || !scale || !Qt || !E || C <= 0 || R <= 0) return MQ_ERR_ARG;
-  if (ldw < R || ldu < C || ld_scale < R) return MQ_ERR_ARG;
-  if (round_dtype < 0 || round_dtype > 2) return MQ_ERR_ARG;
-  if (block <= 0 || block > B) block = B;  // wider blocks only reassociate the trailing sums
-  LoopArgs a{Wt, ldw, C, R, U, ldu, scale, ld_scale, scale_row, qzero, qzero_const, maxq, round_dtype, Qt, E, nullptr, 0};
-  hipStream_t st = (hipStream_t)stream;
-  if (scale_row) return qzero ? run_loop<true, true>(a, block, st) : run_loop<true, false>(a, block, st);
-  return qzero ? run_loop<false, true>(a, block, st) : run_loop<false, false>(a, block, st);
+  return loop_impl(1, &Wt, ldw, C, R, &U, ldu, &scale, ld_scale, &scale_row, &qzero, qzero_const, maxq, round_dtype, block,
+                   &Qt, &E, nullptr, stream);
+}
+
+// `groups` linears of one shape in one sequence of launches (host arrays of device pointers; scale_row / qzero: NULL,
+// or arrays whose entries are all NULL or all set).  More than MAX_GROUP linears run as consecutive batches.
+extern "C" int mq_gptq_loop_grouped(int groups, float* const* Wt, long ldw, int C, int R, const float* const* U, long ldu,
+                                    const float* const* scale, long ld_scale, const int* const* scale_row,
+                                    const float* const* qzero, float qzero_const, float maxq, int round_dtype, int block,
+                                    uint8_t* const* Qt, float* const* E, void* stream) {
+  if (groups < 0 || (groups > 0 && (!Wt || !U || !scale || !Qt || !E))) return MQ_ERR_ARG;
+  for (int g0 = 0; g0 < groups; g0 += MAX_GROUP) {
+    const int cnt = groups - g0 < MAX_GROUP ? groups - g0 : MAX_GROUP;
+    const int rc = loop_impl(cnt, Wt + g0, ldw, C, R, U + g0, ldu, scale + g0, ld_scale, scale_row ? scale_row + g0 : nullptr,
+                             qzero ? qzero + g0 : nullptr, qzero_const, maxq, round_dtype, block, Qt + g0, E + g0, nullptr,
+                             stream);
+    if (rc != MQ_OK) return rc;
+  }
+  return MQ_OK;
+}
+
+// The loop on the Cholesky multipliers F of mq_factor_chol (in U's place) and the original weights W0t (laid out
+// like Wt, read only): same outputs as the classical loop on U up to fp32 rounding.
+extern "C" int mq_gptq_loop_chol_grouped(int groups, float* const* Wt, const float* const* W0t, long ldw, int C, int R,
+                                         const float* const* F, long ldf, const float* const* scale, long ld_scale,
+                                         const int* const* scale_row, const float* const* qzero, float qzero_const,
+                                         float maxq, int round_dtype, int block, uint8_t* const* Qt, float* const* E,
+                                         void* stream) {
+  if (groups < 0 || (groups > 0 && (!Wt || !W0t || !F || !scale || !Qt || !E))) return MQ_ERR_ARG;
+  for (int g0 = 0; g0 < groups; g0 += MAX_GROUP) {
+    const int cnt = groups - g0 < MAX_GROUP ? groups - g0 : MAX_GROUP;
+    const int rc = loop_impl(cnt, Wt + g0, ldw, C, R, F + g0, ldf, scale + g0, ld_scale, scale_row ? scale_row + g0 : nullptr,
+                             qzero ? qzero + g0 : nullptr, qzero_const, maxq, round_dtype, block, Qt + g0, E + g0, W0t + g0,
+                             stream);
+    if (rc != MQ_OK) return rc;
+  }
+  return MQ_OK;
+}
+
+extern "C" int mq_gptq_loop_chol(float* Wt, const float* W0t, long ldw, int C, int R, const float* F, long ldf,
+                                 const float* scale, long ld_scale, const int* scale_row, const float* qzero,
+                                 float qzero_const, float maxq, int round_dtype, int block, uint8_t* Qt, float* E,
+                                 void* stream) {
+  return mq_gptq_loop_chol_grouped(1, &Wt, &W0t, ldw, C, R, &F, ldf, &scale, ld_scale, &scale_row, &qzero, qzero_const, maxq,
+                                   round_dtype, block, &Qt, &E, stream);
 }

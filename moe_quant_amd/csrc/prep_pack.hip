@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void mse_scale_kernel(const void* __restrict__
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void prepare_wt_kernel(const void* __restrict__ W, int wdt, long ldw, int R, int C,
                                                          const int* __restrict__ perm, const uint8_t* __restrict__ dead,
-                                                         float* __restrict__ Wt, long ldwt) {
+                                                         float* __restrict__ Wt, float* __restrict__ Wt2, long ldwt) {
   __shared__ float t[64][65];
   const int j0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
@@ -216,7 +216,10 @@ __global__ __launch_bounds__(256) void prepare_wt_kernel(const void* __restrict_
   }
   __syncthreads();
   for (int jj = ty; jj < 64; jj += 4) {
-    if (j0 + jj < C && r0 + tx < R) Wt[(long)(j0 + jj) * ldwt + r0 + tx] = t[tx][jj];
+    if (j0 + jj < C && r0 + tx < R) {
+      Wt[(long)(j0 + jj) * ldwt + r0 + tx] = t[tx][jj];
+      if (Wt2) Wt2[(long)(j0 + jj) * ldwt + r0 + tx] = t[tx][jj];  // second copy: the loop keeps one read-only
+    }
   }
 }
 
@@ -416,12 +419,17 @@ extern "C" int mq_mse_scale_sym(const void* W, int w_dtype, long ldw, int R, int
   return mq_check_launch();
 }
 
+extern "C" int mq_prepare_wt_pair(const void* W, int w_dtype, long ldw, int R, int C, const int* perm,
+                                  const uint8_t* dead_cols, float* Wt, float* Wt2, long ldwt, void* stream) {
+  if (!W || !Wt || Wt == Wt2 || R <= 0 || C <= 0 || ldw < C || ldwt < R || w_dtype < 0 || w_dtype > 2) return MQ_ERR_ARG;
+  hipLaunchKernelGGL(prepare_wt_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream, W,
+                     w_dtype, ldw, R, C, perm, dead_cols, Wt, Wt2, ldwt);
+  return mq_check_launch();
+}
+
 extern "C" int mq_prepare_wt(const void* W, int w_dtype, long ldw, int R, int C, const int* perm,
                              const uint8_t* dead_cols, float* Wt, long ldwt, void* stream) {
-  if (!W || !Wt || R <= 0 || C <= 0 || ldw < C || ldwt < R || w_dtype < 0 || w_dtype > 2) return MQ_ERR_ARG;
-  hipLaunchKernelGGL(prepare_wt_kernel, dim3((C + 63) / 64, (R + 63) / 64), dim3(256), 0, (hipStream_t)stream, W,
-                     w_dtype, ldw, R, C, perm, dead_cols, Wt, ldwt);
-  return mq_check_launch();
+  return mq_prepare_wt_pair(W, w_dtype, ldw, R, C, perm, dead_cols, Wt, nullptr, ldwt, stream);
 }
 
 extern "C" int mq_untranspose_codes(const uint8_t* Qt, int R, int C, const int* perm_inv, uint8_t* codes, long ldc,

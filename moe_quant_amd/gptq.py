@@ -81,7 +81,8 @@ class GPTQ:
         self._H_clean = False  # H went through the pre-step scan and nothing touched it since (idem)
         # engine state shared with tied handles (the reference recomputes both for every tied handle)
         self._perm = None
-        self._hessian_inv = None
+        self._hessian_inv = None  # U, when somebody asked for it through _get_hessian_inverse
+        self._loop_factor = None  # F, the multipliers the quantize path hands to the loop (kept for tied handles)
 
     # The reference keeps three host booleans and pays a device->host read for two of them inside quantize().
     # Here the verdicts stay on the device (so linears can be queued back to back on several streams) and are
@@ -192,19 +193,19 @@ class GPTQ:
         self.W = self.layer.weight
         if self.num_tied_handles == 0:
             self.H = None
-            self._hessian_inv = None
+            self._hessian_inv = self._loop_factor = None
             self._H_upper_only = self._H_clean = False
         elif self.tied_gptq_handle:
             self.tied_gptq_handle.num_tied_handles -= 1
             if self.tied_gptq_handle.num_tied_handles == 0:
                 self.tied_gptq_handle.H = None
-                self.tied_gptq_handle._hessian_inv = None
+                self.tied_gptq_handle._hessian_inv = self.tied_gptq_handle._loop_factor = None
                 self.tied_gptq_handle._H_upper_only = self.tied_gptq_handle._H_clean = False
         self.num_samples = 0
         self._perm = None
         self._pruned = None
         if self.tied_gptq_handle is not None:
-            self._hessian_inv = None
+            self._hessian_inv = self._loop_factor = None
         torch.cuda.empty_cache()
 
     # ---- pre-step: src/gptq.py:122-154 --------------------------------------------------------------
@@ -249,7 +250,9 @@ class GPTQ:
 
     # ---- quantize: src/gptq.py:156-218 ---------------------------------------------------------------
     @torch.no_grad()
-    def _quantize(self, bits: int) -> Tuple[Tensor, Tensor, Tensor]:
+    def _prepare(self, bits: int) -> dict:
+        """Everything `_quantize` does before the factorisation: scales from the un-updated weights, the column
+        order, H permuted in place of the reference's `H[perm][:, perm]`."""
         if not self.sym:
             raise NotImplementedError("only symmetric quantization is supported (as MoE-Quant's README states)")
         d_col, dtype, device = self.d_col, self.W_dtype, self.W_device
@@ -262,7 +265,7 @@ class GPTQ:
             ops.mse_scale_sym_(W, group_size, points, scale_rg, scale_gr, float(2 ** (bits - 1)), float(2**bits - 1), 2.4,
                                dtype, dead_cols=dead)
         tied = self.tied_gptq_handle
-        perm = perm_inv = perm_i32 = perm_inv_i32 = None
+        perm = perm_i32 = perm_inv_i32 = None
         if self.quantization_order == QuantizationOrder.ACTIVATION:
             if tied is not None and tied._perm is not None:
                 # the owner's H is already permuted; reuse its order (the reference re-sorts the sorted
@@ -275,20 +278,88 @@ class GPTQ:
             self._perm = perm
             if tied is None:
                 self.H = self.H[perm][:, perm]
-        hessian_inv = self._get_hessian_inverse()
-        Wt = ops.prepare_wt(W, perm_i32, dead_cols=dead)
         if perm is None:
             scale_row = torch.arange(d_col, device=device, dtype=torch.int32) // group_size
         else:
             scale_row = (perm // group_size).to(torch.int32)
-        maxq = float(2**bits - 1)
-        qzero = float(2 ** (bits - 1))
-        Qt = ops.gptq_loop_(Wt, hessian_inv, scale_gr, scale_row, None, qzero, maxq, dtype, self.block_size)
-        self._Qt, self._perm_inv_i32 = Qt, perm_inv_i32
-        qweight = ops.untranspose_codes(Qt, perm_inv_i32)
-        scale = scale_rg.to(dtype)
-        zero = torch.full_like(scale, qzero)
+        return dict(W=W, dead=dead, scale_rg=scale_rg, scale_gr=scale_gr, perm_i32=perm_i32, perm_inv_i32=perm_inv_i32,
+                    scale_row=scale_row, maxq=float(2**bits - 1), qzero=float(2 ** (bits - 1)))
+
+    def _finish(self, ctx: dict, Qt: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+        """The reference's post-loop casts (src/gptq.py:199-202)."""
+        self._Qt, self._perm_inv_i32 = Qt, ctx["perm_inv_i32"]
+        qweight = ops.untranspose_codes(Qt, ctx["perm_inv_i32"])
+        scale = ctx["scale_rg"].to(self.W_dtype)
+        zero = torch.full_like(scale, ctx["qzero"])
         return qweight, scale, zero
+
+    @torch.no_grad()
+    def _quantize(self, bits: int) -> Tuple[Tensor, Tensor, Tensor]:
+        return GPTQ._quantize_prepared([self], [self._prepare(bits)])[0]
+
+    @staticmethod
+    def _quantize_prepared(handles, ctxs):
+        """Factorisation, column loop and post-loop casts for handles of one shape whose `_prepare` has run.
+
+        The loop runs in its inverse-free form: with H = R R^T (R upper), the reference's factor is U = R^-1
+        (src/gptq.py:236-242) and its recurrence x_k = w_k + sum_{j<k} e_j U[j,k]/U[j,j] equals
+        x_k = w_k - (1/R_kk) sum_{j<k} z_j R[j,k] with z_j the total change of column j, so only the Cholesky factor
+        is computed (half the flop) and the loop gets F = -R[j,k]/R[k,k] and a copy of the original weights.
+        `_get_hessian_inverse` / `gptq_loop.gptq_loop` keep the reference's U-based forms."""
+        h0 = handles[0]
+        # factors: reuse what tied owners hold, factor the rest side by side
+        need = []
+        for h in handles:
+            tied = h.tied_gptq_handle
+            shares = tied is not None and tied.H is h.H
+            if shares and (tied._loop_factor is not None or any(tied is o for o in need)):
+                continue  # the owner's factor: already there, or computed below
+            h._damp_hessian()
+            need.append(h)
+        own = {}
+        if need:
+            Hs = [o.H for o in need]
+            C = h0.d_col
+            if C % 128 or any(H.dtype != torch.float32 or H.stride(1) != 1 or H.stride(0) != C or H.data_ptr() % 16
+                              for H in Hs):
+                Hs = [linalg_utils._padded_copy(H) for H in Hs]  # identity-padded to a multiple of 128, contiguous
+            Fs, infos = ops.factor_chol_grouped(Hs)
+            GPTQ.factor_calls += len(need)
+            for i, o in enumerate(need):
+                own[id(o)], o._info = Fs[i], infos[i:i + 1]
+                if o.num_tied_handles > 0:
+                    o._loop_factor = Fs[i]
+        Fs = []
+        for h in handles:
+            tied = h.tied_gptq_handle
+            Fs.append(own[id(h)] if id(h) in own else (own[id(tied)] if id(tied) in own else tied._loop_factor))
+        pairs = [ops.prepare_wt_pair(c["W"], c["perm_i32"], dead_cols=c["dead"]) for c in ctxs]
+        Qts = ops.gptq_loop_chol_grouped_([p[0] for p in pairs], [p[1] for p in pairs], Fs, [c["scale_gr"] for c in ctxs],
+                                          [c["scale_row"] for c in ctxs], ctxs[0]["qzero"], ctxs[0]["maxq"], h0.W_dtype,
+                                          h0.block_size)
+        return [h._finish(c, Qt) for h, c, Qt in zip(handles, ctxs, Qts)]
+
+    @staticmethod
+    @torch.no_grad()
+    def quantize_many(handles, bits: int):
+        """`[h.quantize(bits) for h in handles]` for linears of one shape and one configuration (the experts of a
+        block, which the reference quantizes one after another, quant.py:291-386), with the two long phases --
+        factorisation and column loop -- run as one grouped library call each: a lone factorisation or loop is a
+        chain of dependent launches that cannot fill the GPU.  Same results, bit for bit, as one call per handle.
+        A tied handle must come after its owner (in this list or in an earlier call)."""
+        handles = list(handles)
+        if not handles:
+            return []
+        h0 = handles[0]
+        key = lambda h: (h.d_row, h.d_col, h.W_dtype, h.group_size, min(h.block_size, 128), h.sym, h.W_device)
+        if any(key(h) != key(h0) for h in handles):
+            raise ValueError("quantize_many needs linears of one shape, dtype, group size and block size")
+        ctxs = []
+        for h in handles:  # in list order: a tied handle picks up what its owner's steps left (H, column order)
+            h.quantization_pre_step()
+            h._pin_inputs_to_current_stream()
+            ctxs.append(h._prepare(bits))
+        return GPTQ._quantize_prepared(handles, ctxs)
 
     def _kernel_weights(self):
         """(weights, pruned mask) the kernels read: after the pre-step the layer's own weights plus the mask stand
@@ -320,22 +391,29 @@ class GPTQ:
         return ops.pack_from_qt(self._Qt, self._perm_inv_i32)
 
     # ---- inverse factor: src/gptq.py:220-243 ---------------------------------------------------------
+    def _damp_hessian(self) -> None:
+        """All-zero weight columns -> unit rows/columns of H, then damping (src/gptq.py:221-234); a tied handle finds
+        both done by its owner."""
+        if not self.tied_gptq_handle:
+            H = self.H
+            flags = self._flags if self._flags is not None else torch.zeros(4, dtype=torch.int32, device=H.device)
+            w, pruned = self._kernel_weights()
+            ops.hessian_damp_(H, w, pruned, self.rel_damp, flags)
+            self._H_clean = True
+
+    def _factor_hessian(self) -> Tensor:
+        # a failed factorisation yields the identity on the device, the reference's `except` branch
+        # (src/gptq.py:239-240, which never sets issue_non_invertible; this engine does)
+        U, self._info = linalg_utils.inverse_cholesky_factor(self.H)
+        GPTQ.factor_calls += 1
+        if self.num_tied_handles > 0:
+            self._hessian_inv = U
+        return U
+
     @torch.no_grad()
     def _get_hessian_inverse(self) -> Tensor:
         tied = self.tied_gptq_handle
         if tied is not None and tied._hessian_inv is not None and tied.H is self.H:
             return tied._hessian_inv  # same damped H -> same factor; the reference recomputes it
-        H = self.H
-        if not tied:
-            # all-zero weight columns -> unit rows/columns of H, then damping (src/gptq.py:221-234)
-            flags = self._flags if self._flags is not None else torch.zeros(4, dtype=torch.int32, device=H.device)
-            w, pruned = self._kernel_weights()
-            ops.hessian_damp_(H, w, pruned, self.rel_damp, flags)
-            self._H_clean = True
-        # a failed factorisation yields the identity on the device, the reference's `except` branch
-        # (src/gptq.py:239-240, which never sets issue_non_invertible; this engine does)
-        U, self._info = linalg_utils.inverse_cholesky_factor(H)
-        GPTQ.factor_calls += 1
-        if self.num_tied_handles > 0:
-            self._hessian_inv = U
-        return U
+        self._damp_hessian()
+        return self._factor_hessian()

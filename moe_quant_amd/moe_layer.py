@@ -63,14 +63,17 @@ def quantize_moe_layer(
     keep_outputs: bool = False,
     keep_codes: Optional[List[int]] = None,
     max_rows_per_update: int = 1 << 17,
-    streams: int = 4,
+    streams: int = 2,
+    group: int = 8,
 ) -> LayerResult:
     """x (T, C) bf16 on the GPU, expert_ids (T, top_k) int64 on the GPU.
 
-    `streams`: experts are quantized round-robin on that many HIP streams.  One linear is a long chain of
-    dependent launches whose tail (small trailing updates behind one-workgroup diagonal blocks) leaves most
-    of the GPU idle; independent linears on other streams fill it.  Nothing in the per-linear path reads a
-    value back to the host, so one host thread keeps all streams fed."""
+    `group`, `streams`: one linear is a long chain of dependent launches whose critical path (one-workgroup
+    diagonal blocks, 64-row column walks) leaves most of the GPU idle.  Experts are therefore quantized `group` at a
+    time -- their factorisations and column loops run as grouped library calls, every launch carrying the work of
+    all of them -- and the groups go round-robin onto `streams` HIP streams, so that the short per-linear kernels
+    of one group overlap the long launches of another.  Nothing in the path reads a value back to the host, so one
+    host thread keeps all streams fed."""
     dev = x.device
     E = len(experts)
     keep_codes = set(keep_codes or [])
@@ -121,18 +124,29 @@ def quantize_moe_layer(
             s_.wait_stream(main)
     done = []  # (name, handle): verdict words are read after everything is queued
     factor_calls_before = GPTQ.factor_calls
-    for e, (g, u, d) in enumerate(handles):
-        lane = lanes[e % len(lanes)]
+    group = max(1, group)
+    for ci, e0 in enumerate(range(0, E, group)):
+        chunk = list(range(e0, min(E, e0 + group)))
+        lane = lanes[ci % len(lanes)]
         with torch.cuda.stream(lane):
-            if e in keep_codes:
-                g.symmetrize_hessian()
-                d.symmetrize_hessian()
-                if g.H is not None:
-                    res.hessians[f"{e}.gate_proj"] = g.H.clone()
-                if d.H is not None:
-                    res.hessians[f"{e}.down_proj"] = d.H.clone()
-            for name, h in (("gate_proj", g), ("up_proj", u), ("down_proj", d)):
-                q, s, z = h.quantize(bits)
+            for e in chunk:
+                g, u, d = handles[e]
+                if e in keep_codes:
+                    g.symmetrize_hessian()
+                    d.symmetrize_hessian()
+                    if g.H is not None:
+                        res.hessians[f"{e}.gate_proj"] = g.H.clone()
+                    if d.H is not None:
+                        res.hessians[f"{e}.down_proj"] = d.H.clone()
+            # gate and up projections of the chunk (one factor per expert, shared), then the down projections
+            gu = [handles[e][i] for e in chunk for i in (0, 1)]
+            names = [(e, n) for e in chunk for n in ("gate_proj", "up_proj")] + [(e, "down_proj") for e in chunk]
+            dn = [handles[e][2] for e in chunk]
+            if group > 1:
+                outs = GPTQ.quantize_many(gu, bits) + GPTQ.quantize_many(dn, bits)
+            else:
+                outs = [h.quantize(bits) for h in gu + dn]
+            for (e, name), h, (q, s, z) in zip(names, gu + dn, outs):
                 words = h.packed_words()
                 done.append((f"{e}.{name}", h))
                 if keep_outputs:
@@ -141,11 +155,9 @@ def quantize_moe_layer(
                 if e in keep_codes:
                     res.qweight[f"{e}.{name}"] = q
                     res.scales[f"{e}.{name}"] = s
-            for h in (g, u, d):  # as quant.py:330: free per-linear state as soon as the linear is done
-                if h.H is not None and lane is not main:
-                    h.H.record_stream(lane)  # allocated on the main stream, last used on this one
+            for h in gu + dn:  # as quant.py:330: free per-linear state as soon as the linear is done
                 h.H = None
-                h._hessian_inv = None
+                h._hessian_inv = h._loop_factor = None
                 h._Qt = None
                 h.W = h.layer.weight
     for s_ in lanes:

@@ -206,6 +206,69 @@ def factor_upper_inverse_from(H: Tensor, info: Optional[Tensor] = None, normaliz
     return U, info
 
 
+def _ptr_array(tensors):
+    import ctypes as C_
+
+    return (C_.c_void_p * len(tensors))(*[None if t is None else t.data_ptr() for t in tensors])
+
+
+def factor_upper_inverse_from_grouped(Hs, normalize: bool = True):
+    """factor_upper_inverse_from for several matrices of one size with one library call: returns (Us, infos), infos a
+    device int32 vector with one word per matrix.  Bit-identical to separate calls."""
+    _dev(*Hs)
+    lib = _lib.load()
+    k = len(Hs)
+    if k == 0:
+        return [], None
+    C = Hs[0].shape[0]
+    ld = Hs[0].stride(0)
+    for H in Hs:
+        if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1 or C % 128 or H.stride(0) != ld:
+            raise ValueError("every H must be (C,C) fp32 with unit column stride, one pitch, C % 128 == 0")
+    infos = torch.zeros(k, dtype=torch.int32, device=Hs[0].device)
+    Us = [torch.empty((C, C), dtype=torch.float32, device=Hs[0].device) for _ in range(k)]
+    import ctypes as C_
+
+    ip = (C_.c_void_p * k)(*[infos.data_ptr() + 4 * i for i in range(k)])
+    rc = lib.mq_factor_upper_inverse_grouped(k, _ptr_array(Hs), ld, _ptr_array(Us), C, C, int(normalize), ip, _stream(Hs[0]))
+    check(rc, "mq_factor_upper_inverse_grouped")
+    return Us, infos
+
+
+def factor_chol_grouped(Hs):
+    """Cholesky-only factorisation of several matrices of one size with one library call: returns (Fs, infos) with
+    F[j,k] = -R[j,k]/R[k,k] above the diagonal (H = R R^T), the multipliers of gptq_loop_chol_; the diagonal and
+    the lower triangle of every F are undefined.  Bit-identical to separate calls."""
+    _dev(*Hs)
+    lib = _lib.load()
+    k = len(Hs)
+    if k == 0:
+        return [], None
+    C = Hs[0].shape[0]
+    ld = Hs[0].stride(0)
+    for H in Hs:
+        if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1 or C % 128 or H.stride(0) != ld:
+            raise ValueError("every H must be (C,C) fp32 with unit column stride, one pitch, C % 128 == 0")
+    dev = Hs[0].device
+    infos = torch.zeros(k, dtype=torch.int32, device=dev)
+    Fs = [torch.empty((C, C), dtype=torch.float32, device=dev) for _ in range(k)]
+    need = lib.mq_factor_chol_workspace_bytes(C)
+    ws = _ws.get(dev, need * k, "chol")
+    import ctypes as C_
+
+    ip = (C_.c_void_p * k)(*[infos.data_ptr() + 4 * i for i in range(k)])
+    wp = (C_.c_void_p * k)(*[ws.data_ptr() + need * i for i in range(k)])
+    rc = lib.mq_factor_chol_grouped(k, _ptr_array(Hs), ld, _ptr_array(Fs), C, C, ip, wp, need, _stream(Hs[0]))
+    check(rc, "mq_factor_chol_grouped")
+    return Fs, infos
+
+
+def factor_chol(H: Tensor):
+    """(F, info) for one matrix, see factor_chol_grouped."""
+    Fs, infos = factor_chol_grouped([H])
+    return Fs[0], infos
+
+
 # ---- (3) grid, layout, loop --------------------------------------------------------------------------
 def quant_grid_sym(W: Tensor, group_size: int, bits: int, round_dtype, dead_cols: Optional[Tensor] = None,
                    want_transposed: bool = True) -> Tuple[Tensor, Optional[Tensor]]:
@@ -258,6 +321,60 @@ def prepare_wt(W: Tensor, perm: Optional[Tensor] = None, dead_cols: Optional[Ten
     return Wt
 
 
+def prepare_wt_pair(W: Tensor, perm: Optional[Tensor] = None, dead_cols: Optional[Tensor] = None):
+    """prepare_wt twice: (Wt, W0t), the copy the loop updates in place and the copy it keeps reading."""
+    _dev(W, perm, dead_cols)
+    lib = _lib.load()
+    R, C = W.shape
+    if W.stride(1) != 1:
+        W = W.contiguous()
+    Wt = torch.empty(C, R, dtype=torch.float32, device=W.device)
+    W0t = torch.empty(C, R, dtype=torch.float32, device=W.device)
+    rc = lib.mq_prepare_wt_pair(W.data_ptr(), _dt(W.dtype), W.stride(0), R, C, _p(perm), _p(dead_cols), Wt.data_ptr(),
+                                W0t.data_ptr(), R, _stream(W))
+    check(rc, "mq_prepare_wt_pair")
+    return Wt, W0t
+
+
+def gptq_loop_chol_grouped_(Wts, W0ts, Fs, scales, scale_rows, qzero_const: float, maxq: float, round_dtype, block: int):
+    """The inverse-free loop for several linears of one shape with one library call: Fs from factor_chol_grouped,
+    (Wts, W0ts) from prepare_wt_pair.  In place on every Wt; returns the list of code tensors Qt (C,R) uint8."""
+    k = len(Wts)
+    if not (len(W0ts) == len(Fs) == len(scales) == k) or (scale_rows is not None and len(scale_rows) != k):
+        raise ValueError("Wts, W0ts, Fs, scales, scale_rows must have the same length")
+    if k == 0:
+        return []
+    _dev(*Wts, *W0ts, *Fs, *scales, *(scale_rows or []))
+    lib = _lib.load()
+    C, R = Wts[0].shape
+    ldw, ldf, lds = Wts[0].stride(0), Fs[0].stride(0), scales[0].stride(0)
+    for Wt, W0t, F, sc in zip(Wts, W0ts, Fs, scales):
+        for t in (Wt, W0t, F, sc):
+            if t.dtype != torch.float32 or t.stride(-1) != 1:
+                raise ValueError("Wt, W0t, F, scale must be fp32 with unit inner stride")
+        if (Wt.shape != (C, R) or W0t.shape != (C, R) or Wt.stride(0) != ldw or W0t.stride(0) != ldw or F.stride(0) != ldf
+                or sc.stride(0) != lds):
+            raise ValueError("all linears of a group share one shape and one set of pitches")
+    if scale_rows is not None:
+        for m in scale_rows:
+            if m.dtype != torch.int32 or m.numel() != C:
+                raise ValueError("scale_row must be int32 of length C")
+    elif scales[0].shape[0] != C:
+        raise ValueError("scale must be (C,R) when no scale_row map is given")
+    dev = Wts[0].device
+    Qts = [torch.empty(C, R, dtype=torch.uint8, device=dev) for _ in range(k)]
+    ring = 8 * 128 * R * 4
+    E = _ws.get(dev, ring * k, "loop")
+    import ctypes as C_
+
+    Ep = (C_.c_void_p * k)(*[E.data_ptr() + ring * i for i in range(k)])
+    rc = lib.mq_gptq_loop_chol_grouped(k, _ptr_array(Wts), _ptr_array(W0ts), ldw, C, R, _ptr_array(Fs), ldf,
+                                       _ptr_array(scales), lds, _ptr_array(scale_rows) if scale_rows is not None else None,
+                                       None, qzero_const, maxq, _dt(round_dtype), block, _ptr_array(Qts), Ep, _stream(Wts[0]))
+    check(rc, "mq_gptq_loop_chol_grouped")
+    return Qts
+
+
 def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor], qzero: Optional[Tensor],
                qzero_const: float, maxq: float, round_dtype, block: int) -> Tensor:
     """Runs the loop in place on Wt (C,R); returns the codes Qt (C,R) uint8."""
@@ -280,6 +397,44 @@ def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor]
                           Qt.data_ptr(), E.data_ptr(), _stream(Wt))
     check(rc, "mq_gptq_loop")
     return Qt
+
+
+def gptq_loop_grouped_(Wts, Us, scales, scale_rows, qzero_const: float, maxq: float, round_dtype, block: int):
+    """gptq_loop_ for several linears of one shape with one library call (lists of equal length; scale_rows: a list of
+    int32 maps or None).  In place on every Wt; returns the list of code tensors Qt (C,R) uint8."""
+    k = len(Wts)
+    if not (len(Us) == len(scales) == k) or (scale_rows is not None and len(scale_rows) != k):
+        raise ValueError("Wts, Us, scales, scale_rows must have the same length")
+    if k == 0:
+        return []
+    _dev(*Wts, *Us, *scales, *(scale_rows or []))
+    lib = _lib.load()
+    C, R = Wts[0].shape
+    ldw, ldu, lds = Wts[0].stride(0), Us[0].stride(0), scales[0].stride(0)
+    for Wt, U, sc in zip(Wts, Us, scales):
+        for t in (Wt, U, sc):
+            if t.dtype != torch.float32 or t.stride(-1) != 1:
+                raise ValueError("Wt, U, scale must be fp32 with unit inner stride")
+        if Wt.shape != (C, R) or Wt.stride(0) != ldw or U.stride(0) != ldu or sc.stride(0) != lds:
+            raise ValueError("all linears of a group share one shape and one set of pitches")
+    if scale_rows is not None:
+        for m in scale_rows:
+            if m.dtype != torch.int32 or m.numel() != C:
+                raise ValueError("scale_row must be int32 of length C")
+    elif scales[0].shape[0] != C:
+        raise ValueError("scale must be (C,R) when no scale_row map is given")
+    dev = Wts[0].device
+    Qts = [torch.empty(C, R, dtype=torch.uint8, device=dev) for _ in range(k)]
+    ring = 8 * 128 * R * 4
+    E = _ws.get(dev, ring * k, "loop")
+    import ctypes as C_
+
+    Ep = (C_.c_void_p * k)(*[E.data_ptr() + ring * i for i in range(k)])
+    rc = lib.mq_gptq_loop_grouped(k, _ptr_array(Wts), ldw, C, R, _ptr_array(Us), ldu, _ptr_array(scales), lds,
+                                  _ptr_array(scale_rows) if scale_rows is not None else None, None, qzero_const, maxq,
+                                  _dt(round_dtype), block, _ptr_array(Qts), Ep, _stream(Wts[0]))
+    check(rc, "mq_gptq_loop_grouped")
+    return Qts
 
 
 def untranspose_codes(Qt: Tensor, perm_inv: Optional[Tensor] = None) -> Tensor:

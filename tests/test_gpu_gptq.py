@@ -203,6 +203,25 @@ def test_model_dtypes_of_the_reference_driver(dev, wdt, xdt):
     _run_case(case, dev, chunks=2)
 
 
+def test_block_size_none_means_whole_width(dev):
+    """GPTQ(block_size=None) is block = d_col in the reference (src/gptq.py:45): every error goes into every later
+    column at once, no lazy batches.  The engine walks 128 columns at a time whatever the block argument says, which
+    only changes the order of the fp32 sums: codes against the oracle run at block = C."""
+    case = synth.config1(0.125)
+    case.block_size = None
+    h = GPTQ(_layer(case.W, dev), group_size=128, sym=True, rel_damp=0.01, block_size=None)
+    assert h.block_size == case.W.shape[1]
+    h.update(case.X.to(dev))
+    q, s, z = h.quantize(4)
+    Href, _ = O.hessian_update(None, 0, case.X)
+    ref = O.quantize_linear(case.W, Href, block_size=None)
+    ref128 = O.quantize_linear(case.W, Href.clone(), block_size=128)
+    m, m128 = [(q.cpu() == r["qweight"]).float().mean().item() for r in (ref, ref128)]
+    own = (ref["qweight"] == ref128["qweight"]).float().mean().item()
+    _say(f"block=None: match vs oracle(block=C) {m:.6f}, vs oracle(block=128) {m128:.6f}; oracle C vs 128 {own:.6f}")
+    assert torch.equal(s.cpu(), ref["scale"]) and m >= 0.999 and m128 >= 0.999
+
+
 def test_nan_hessian_falls_back(dev):
     W = synth.weight(64, 256, 2)
     h = GPTQ(_layer(W, dev), 128, True)
@@ -357,3 +376,28 @@ def test_pack_weight_accepts_cpu_tensors_like_the_reference_cli(dev):
     out = pack_weight({"qweight": q, "scale": s, "zero": z}, 4, True, 128)
     assert out["weight_packed"].device.type == "cpu"
     assert torch.equal(out["weight_packed"], O.pack_to_int32(q.to(torch.int8) - 8, 4))
+
+
+@pytest.mark.parametrize("act_order", [False, True])
+def test_quantize_many_equals_one_at_a_time(dev, act_order):
+    """Grouped factorisation + grouped loop through the handle API: gate/up pairs (tied) of four experts, against the
+    same handles quantized one by one."""
+    order = "activation" if act_order else "default"
+    R, C, n = 256, 640, 900
+
+    def make():
+        hs = []
+        for e in range(4):
+            g = GPTQ(_layer(synth.weight(R, C, 40 + 2 * e), dev), 128, True, 0.01, 128, quantization_order=order)
+            u = GPTQ(_layer(synth.weight(R, C, 41 + 2 * e), dev), 128, True, 0.01, 128, quantization_order=order,
+                     tied_gptq_handle=g)
+            g.update(synth.activations_outlier(n + 64 * e, C, 60 + e).to(dev))
+            hs += [g, u]
+        return hs
+
+    before = GPTQ.factor_calls
+    many = GPTQ.quantize_many(make(), 4)
+    assert GPTQ.factor_calls - before == 4  # one factor per gate/up pair
+    singles = [h.quantize(4) for h in make()]
+    for i, ((q, s, z), (q1, s1, z1)) in enumerate(zip(many, singles)):
+        assert torch.equal(q, q1) and torch.equal(s, s1) and torch.equal(z, z1), i
