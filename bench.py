@@ -44,6 +44,23 @@ def parse():
     return ap.parse_args()
 
 
+def traffic_from_profiles(call, **keys):
+    """HBM bytes per call of `call` for the configuration `keys`, from the table of measured traffic committed in
+    profiles/hbm_traffic.md (lines of the form `| call | C=7168 G=8 panels=4 | 1.23e9 | ...`); None if absent."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+    if not os.path.exists(path):
+        return None
+    want = " ".join(f"{k}={v}" for k, v in keys.items())
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 3 and cells[0] == call and cells[1] == want:
+            try:
+                return float(cells[2])
+            except ValueError:
+                return None
+    return None
+
+
 def moe_layer_run(args, with_cpu_oracle=True):
     """Config 3: every Hessian of a DeepSeek-V3-shaped MoE layer accumulated, 3 linears per expert quantized
     and packed, on one GPU, one pass.  Returns a dict of wall seconds, sizes and (optionally) the parity of the
@@ -229,15 +246,20 @@ def main():
         ops.factor_upper_inverse_(A, info)
 
     t_copy = timed(lambda: A.copy_(Hd), reps=8)
-    t_factor = timed(factor, reps=8) - t_copy
+    t_factor_inv = timed(factor, reps=8) - t_copy  # the reference's factor U (public _get_hessian_inverse path)
+    # what the quantize path runs: the Cholesky factor alone, as the multipliers of the inverse-free loop
+    t_factor = timed(lambda: ops.factor_chol(Hd), reps=8)
+    F, _ = ops.factor_chol(Hd)
     Wd = layer.weight.data
     s_rg, s_gr = ops.quant_grid_sym(Wd, 128, 4, torch.bfloat16)
     scale_row = torch.arange(C, device=dev, dtype=torch.int32) // 128
     Wt0 = ops.prepare_wt(Wd)
     Wt = torch.empty_like(Wt0)
     t_wcopy = timed(lambda: Wt.copy_(Wt0))
-    t_loop = timed(lambda: (Wt.copy_(Wt0), ops.gptq_loop_(Wt, A, s_gr, scale_row, None, 8.0, 15.0, torch.bfloat16, 128))) - t_wcopy
-    Qt = ops.gptq_loop_(Wt, A, s_gr, scale_row, None, 8.0, 15.0, torch.bfloat16, 128)
+    loop1 = lambda: ops.gptq_loop_chol_grouped_([Wt], [Wt0], [F], [s_gr], [scale_row], 8.0, 15.0, torch.bfloat16, 128)[0]
+    t_loop = timed(lambda: (Wt.copy_(Wt0), loop1())) - t_wcopy
+    Wt.copy_(Wt0)
+    Qt = loop1()
     t_pack = timed(lambda: ops.pack_from_qt(Qt), reps=10)
     codes = ops.untranspose_codes(Qt)
     t_pack_rc = timed(lambda: ops.pack_int4(codes), reps=10)
@@ -249,14 +271,14 @@ def main():
     t_syrk_g = timed(lambda: ops.hessian_syrk_grouped_(Hs, [X] * Gq, [0.0] * Gq, [2.0 / n] * Gq, mirror=False)) / Gq
     del Hs
     Hds = [Hd.clone() for _ in range(Gq)]
-    t_factor_g = timed(lambda: ops.factor_upper_inverse_from_grouped(Hds), reps=4) / Gq
+    t_factor_g = timed(lambda: ops.factor_chol_grouped(Hds), reps=4) / Gq
     del Hds
     Wts = [torch.empty_like(Wt0) for _ in range(Gq)]
 
     def loop_grouped():
         for w in Wts:
             w.copy_(Wt0)
-        ops.gptq_loop_grouped_(Wts, [A] * Gq, [s_gr] * Gq, [scale_row] * Gq, 8.0, 15.0, torch.bfloat16, 128)
+        ops.gptq_loop_chol_grouped_(Wts, [Wt0] * Gq, [F] * Gq, [s_gr] * Gq, [scale_row] * Gq, 8.0, 15.0, torch.bfloat16, 128)
 
     t_loop_g = timed(loop_grouped) / Gq - t_wcopy
     del Wts
@@ -267,12 +289,13 @@ def main():
     t_mse = timed(lambda: ops.mse_scale_sym_(Wd, 128, pts, s_try, None, 8.0, 15.0, 2.4, torch.bfloat16))
 
     flop_syrk = n * C * (C + 1)
-    flop_factor = (2.0 / 3.0) * C**3
+    flop_factor = (1.0 / 3.0) * C**3  # one Cholesky factorisation: all the quantize path needs (no inverse)
     flop_loop = R * C * (C - 1)
     bytes_pack = 1.5 * R * C
     phases = {
         "hessian_syrk_ms": round(t_syrk, 4),
         "factor_ms": round(t_factor, 4),
+        "factor_with_inverse_ms_not_in_step": round(t_factor_inv, 4),
         "gptq_loop_ms": round(t_loop, 4),
         "pack_from_loop_codes_ms": round(t_pack, 4),
         "pack_int4_ms": round(t_pack_rc, 4),
@@ -291,24 +314,27 @@ def main():
         "pack_int4_gbps": round(bytes_pack / t_pack_rc / 1e6, 1),
         "pack_int4_frac_hbm_peak": round(bytes_pack / t_pack_rc / 1e6 / PEAK_HBM, 4),
     }
-    # dominant kernel of the step: the factorisation chain (fp32 MFMA bound); achieved = algorithmic
-    # (2/3) C^3 flop / measured device time of the chain
-    # HBM bytes per factorisation of a 7168^2 matrix, from the two rocprofv3 --pmc runs summarised in
-    # profiles/config1_bench_hbm_traffic.md (2.00*FETCH_SIZE + 1.00*WRITE_SIZE, calibrated on copy/fill kernels)
-    traffic = 7.34e9 if C == 7168 else None
+    # Dominant call of the step: the factorisation, as the step runs it -- one grouped call over `group` matrices
+    # (one "launch" = one call = a fixed sequence of kernels, each carrying the work of all matrices).
+    # achieved = algorithmic flop (one Cholesky factorisation per matrix, C^3/3) / device time of the call, measured
+    # above with HIP events on the launch stream.  traffic = HBM bytes per call from the rocprofv3 --pmc runs
+    # summarised in profiles/ (looked up by matrix size, group size and panel batch; null when that table has no
+    # line for this configuration).
+    panels = int(os.environ.get("MQ_PANELS", "4") or 4)
+    traffic = traffic_from_profiles("mq_factor_chol_grouped", C=C, G=Gq, panels=panels)
     roofline = {
-        "kernel": "mq_factor_upper_inverse = trail_diag_kernel + panel_inv_kernel + inv_first_kernel + revchol_diag_kernel + "
-                  "unit_diag_kernel (one launch sequence per call; largest share of the step). fp32 in, fp32 out; the "
+        "kernel": f"mq_factor_chol_grouped over {Gq} matrices = trail_diag_kernel + panel_inv_kernel + revchol_diag_kernel + "
+                  "chol_finalize_kernel (one launch sequence per call; largest share of the step). fp32 in, fp32 out; the "
                   "interior GEMM tiles form each fp32 product from six bf16-piece products on the bf16 matrix cores, so the "
                   "fp32 MFMA figure is the yardstick for the algorithmic flop, not a ceiling of the kernel",
         "bound": "mfma",
-        "achieved": round(flop_factor / t_factor / 1e9, 3),
+        "achieved": round(flop_factor / t_factor_g / 1e9, 3),
         "peak": PEAK_FP32_MFMA,
         "unit": "TFLOP/s",
-        "frac": round(flop_factor / t_factor / 1e9 / PEAK_FP32_MFMA, 4),
+        "frac": round(flop_factor / t_factor_g / 1e9 / PEAK_FP32_MFMA, 4),
         "traffic": traffic,
-        "algorithmic_flop_per_launch": flop_factor,
-        "ms_per_launch": round(t_factor, 4),
+        "algorithmic_flop_per_launch": flop_factor * Gq,
+        "ms_per_launch": round(t_factor_g * Gq, 4),
     }
 
     cpu = None
@@ -340,7 +366,7 @@ def main():
     # the third number of the headline metric: one pass over the whole MoE layer (config 3), outside the timed steps
     moe = None
     if not args.no_moe_layer and args.scale == 1.0:
-        del H, Hd, A, Wt, Wt0, Qt, codes, X
+        del H, Hd, A, F, Wt, Wt0, Qt, codes, X
         torch.cuda.empty_cache()
         moe = moe_layer_run(args, with_cpu_oracle=not args.no_cpu_baseline)
         phases["moe_layer_wall_s"] = moe["wall_s"]

@@ -100,6 +100,12 @@ size_t mq_hessian_damp_workspace_bytes(int C);
 int mq_hessian_damp(float* H, long ldh, int C, const void* W, int w_dtype, long ldw, int R, const uint8_t* pruned,
                     float rel_damp, int* flags, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Activation order: Hp[i, j] = H[perm[i], perm[j]].  Replaces `self.H = self.H[perm][:, perm]`, src/gptq.py:187
+ * (perm = argsort(diag(H), descending), src/gptq.py:181), in one pass and without the intermediate the two chained
+ * gathers build.  H (C x C, ldh) is read only, Hp (C x C, ldp) must not alias it; perm: C int32 on the device.
+ * C <= 40960 (a source row passes through LDS), otherwise MQ_ERR_TOO_LARGE. */
+int mq_permute_symmetric(const float* H, long ldh, const int* perm, float* Hp, long ldp, int C, void* stream);
+
 /* mq_hessian_damp without a workspace argument and without any allocation.  It has no counterpart in MoE-Quant: it
  * exists for callers that cannot allocate or pass scratch memory -- code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  Same arguments, same kernels and bit-identical results; the scratch area

@@ -23,6 +23,7 @@ SIGNATURES = {
     "mq_hessian_syrk_bf16_grouped": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _sz, _vp]),
     "mq_symmetrize_upper": (_i, [_vp, _l, _i, _vp]),
     "mq_hessian_prestep": (_i, [_vp, _l, _i, _i, _vp, _vp, _vp]),
+    "mq_permute_symmetric": (_i, [_vp, _l, _vp, _vp, _l, _i, _vp]),
     "mq_hessian_damp_workspace_bytes": (_sz, [_i]),
     "mq_hessian_damp": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp, _sz, _vp]),
     "mq_hessian_damp_noalloc": (_i, [_vp, _l, _i, _vp, _i, _l, _i, _vp, _f, _vp, _vp]),

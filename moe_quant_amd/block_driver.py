@@ -8,8 +8,9 @@ Given one transformer block already on the device and its calibration inputs it
   4. reports the three issue counters (:332-337, :398-403).
 `save_metadata` writes `<save_dir>/metadata.pt` (:428-435); `get_resume_block_idx` is :91-97.
 
-What differs from the reference, on purpose: linears are queued round-robin on HIP streams and nothing is read
-back while they are queued (the finite check, the issue flags and the files come after one synchronisation);
+What differs from the reference, on purpose: linears of one shape (the experts) are quantized `group` at a time
+through grouped library calls, the groups are queued round-robin on HIP streams, and nothing is read back while
+they are queued (the finite check, the issue flags and the files come after one synchronisation);
 handles are released without `torch.cuda.empty_cache()`.  Model loading, dataset handling, the distributed
 expert split and wandb logging are not part of this engine."""
 from __future__ import annotations
@@ -82,7 +83,8 @@ def quantize_block(
     tie_gptq_handles: bool = False,
     save_dir: Optional[str] = None,
     log_error: bool = False,
-    streams: int = 4,
+    streams: int = 2,
+    group: int = 8,
 ) -> BlockReport:
     """`model`: any module whose linears under `prefix` are to be quantized (names as in `named_modules()`).
     `run_block()`: runs the block once over every calibration sequence (what quant.py:280-281 does); the forward
@@ -120,6 +122,8 @@ def quantize_block(
     main = torch.cuda.current_stream(dev)
     lanes = [main] + [torch.cuda.Stream(device=dev) for _ in range(max(1, streams) - 1)]
 
+    group_size_ = group
+
     def run_group(group: Dict[str, GPTQ], counters: Dict[str, int]) -> None:
         for ln in lanes:
             if ln is not main:
@@ -139,22 +143,27 @@ def quantize_block(
                     units[unit_of[id(t)]].append(name)
                 else:  # its owner belongs to the other group and is finished already
                     units.append([name])
-        for i, unit in enumerate(units):
+        # units of one shape and configuration share grouped library calls, `group` units at a time
+        buckets: Dict[tuple, List[List[str]]] = {}
+        for unit in units:
+            h = group[unit[0]]
+            buckets.setdefault((h.d_row, h.d_col, h.W_dtype, h.W_device), []).append(unit)
+        batches = [b[i:i + max(1, group_size_)] for b in buckets.values() for i in range(0, len(b), max(1, group_size_))]
+        for i, batch in enumerate(batches):
             lane = lanes[i % len(lanes)]
             with torch.cuda.stream(lane):
-                for name in unit:
+                names = [name for unit in batch for name in unit]
+                outs = GPTQ.quantize_many([group[n] for n in names], bits)
+                for name, (qweight, scale, zero) in zip(names, outs):
                     h = group[name]
-                    qweight, scale, zero = h.quantize(bits)
                     deq = quant_utils.dequantize_linear_weight(qweight, scale, zero)
                     err = None
                     if log_error:
                         err = quant_utils.get_relative_mse_error(deq.float(), h.layer.weight.float(), h.H)
                     results[name] = (qweight, scale, zero, deq, torch.isfinite(deq).all(), err)
                     h.layer.weight.data = deq  # quant.py:328
-                for name in unit:  # release the handle's state (reset() without emptying the allocator cache)
+                for name in names:  # release the handle's state (reset() without emptying the allocator cache)
                     h = group[name]
-                    if h.H is not None and lane is not main:
-                        h.H.record_stream(lane)
                     h.H = None
                     h._hessian_inv = h._loop_factor = None
                     h._Qt = None

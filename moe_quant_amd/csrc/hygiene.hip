@@ -184,7 +184,40 @@ __global__ __launch_bounds__(256) void damp_apply_kernel(float* __restrict__ H, 
   if (threadIdx.x == 0) row[r] = (rdead ? 1.f : row[r]) + damp_in[0];
 }
 
+// Hp[i, j] = H[perm[i], perm[j]]: one workgroup per output row.  The source row travels to LDS with coalesced
+// loads, the column gather happens there, the output row leaves coalesced: C^2 floats read, C^2 written, no
+// second intermediate (torch's H[perm][:, perm] builds two).
+__global__ __launch_bounds__(256) void permute_sym_kernel(const float* __restrict__ H, long ldh, const int* __restrict__ perm,
+                                                          float* __restrict__ Hp, long ldp, int C) {
+  extern __shared__ __attribute__((aligned(16))) float prow[];
+  const int i = blockIdx.x;
+  const float* src = H + (long)perm[i] * ldh;
+  for (int k = threadIdx.x; k < C; k += 256) prow[k] = src[k];
+  __syncthreads();
+  float* dst = Hp + (long)i * ldp;
+  for (int j = threadIdx.x; j < C; j += 256) dst[j] = prow[perm[j]];
+}
+
 }  // namespace
+
+extern "C" int mq_permute_symmetric(const float* H, long ldh, const int* perm, float* Hp, long ldp, int C, void* stream) {
+  if (!H || !perm || !Hp || H == Hp || C <= 0 || ldh < C || ldp < C) return MQ_ERR_ARG;
+  const size_t smem = (size_t)C * sizeof(float);
+  if (smem > 160 * 1024) return MQ_ERR_TOO_LARGE;  // one source row must fit the 160 KB of LDS
+  static std::mutex mu;
+  static size_t allowed = 48 * 1024;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (smem > allowed) {
+      if (hipFuncSetAttribute((const void*)permute_sym_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
+          hipSuccess)
+        return MQ_ERR_LAUNCH;
+      allowed = smem;
+    }
+  }
+  hipLaunchKernelGGL(permute_sym_kernel, dim3(C), dim3(256), smem, (hipStream_t)stream, H, ldh, perm, Hp, ldp, C);
+  return mq_check_launch();
+}
 
 extern "C" int mq_hessian_prestep(float* H, long ldh, int C, int upper_only, uint8_t* pruned, int* flags, void* stream) {
   if (!H || !pruned || !flags || C <= 0 || ldh < C) return MQ_ERR_ARG;

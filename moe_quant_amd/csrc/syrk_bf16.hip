@@ -211,28 +211,10 @@ __global__ __launch_bounds__(256) void syrk_reduce_kernel(float* __restrict__ H,
 }
 
 // =============================================================================================
-// Large-tile kernel: 256x256 channels per workgroup, four wavefronts of 128x128 (4x4 MFMA blocks,
-// 256 accumulator registers each).  With 64x64 per wave every MFMA needs 0.5 LDS fragment reads;
-// 128x128 per wave needs 0.25, which leaves the LDS port room for the staging writes.
-//
-// Staging: 64 tokens per stage.  Each thread owns two 8-channel x 8-token patches per stage: eight
-// 16-byte loads each (32 lanes side by side read 512 contiguous bytes of one token row), an 8x8
-// transpose in registers (32 byte permutes) and eight 16-byte LDS writes, one per channel.
-// LDS layout per operand: [token octet][channel] in 16-byte chunks (the 8 tokens of one channel), with
-// one spare chunk after every 8 channels.  A fragment read (32 consecutive channels, one token octet)
-// is then a contiguous run of chunks, and the eight lanes that write the same channel-within-octet land
-// 9 chunks apart: both directions are free of bank conflicts.
-// The next stage's 16 loads per thread are in flight during the whole current stage.
+// Large tiles: 256x256 channels per workgroup.
 // =============================================================================================
 constexpr int T2 = 256;
-constexpr int KT2 = 64;                               // tokens per stage
-constexpr int OCT_CHUNKS = T2 + T2 / 8;               // chunks per token octet (with the spare ones)
-constexpr int OP_ELEMS = (KT2 / 8) * OCT_CHUNKS * 8;  // bf16 elements per operand tile
-constexpr size_t BIG_SMEM = (size_t)2 * 2 * OP_ELEMS * sizeof(uint16_t);
-
-__device__ __forceinline__ int chunk_of(int oct, int ch) { return oct * OCT_CHUNKS + ch + (ch >> 3); }
-
-// Tile order for the big kernel.  Upper-triangle tiles are enumerated super-tile by super-tile
+// Tile order for the 256x256 kernel.  Upper-triangle tiles are enumerated super-tile by super-tile
 // (4 row tiles x 8 column tiles): the ~32 workgroups an XCD runs at any moment then touch about a dozen
 // distinct channel panels instead of ~30, so more of their loads hit that XCD's L2.
 __device__ __forceinline__ void blocked_tri_decode(int L, int T, int& tm, int& tn) {
@@ -265,154 +247,6 @@ __device__ __forceinline__ void blocked_tri_decode(int L, int T, int& tm, int& t
     }
   }
   tm = tn = 0;  // not reached for L < T(T+1)/2
-}
-
-struct Patch8 {
-  uint4 r[8];  // r[t] = 8 channels of token t0+t
-  // GUARD = false: the caller knows all 8 tokens and 8 channels are in range (no per-load branch)
-  template <bool GUARD>
-  __device__ __forceinline__ void load(const uint16_t* __restrict__ X, long ldx, int t0, int tend, int c, int C) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (GUARD) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (t0 + i < tend && c < C) v = *reinterpret_cast<const uint4*>(X + (long)(t0 + i) * ldx + c);
-        r[i] = v;
-      } else {
-        r[i] = *reinterpret_cast<const uint4*>(X + (long)(t0 + i) * ldx + c);
-      }
-    }
-  }
-  // writes channel rows ch..ch+7 (ch a multiple of 8) of token octet `oct` of an operand tile
-  __device__ __forceinline__ void store(uint16_t* __restrict__ tile, int ch, int oct) const {
-    const uint32_t in[8][4] = {{r[0].x, r[0].y, r[0].z, r[0].w}, {r[1].x, r[1].y, r[1].z, r[1].w},
-                               {r[2].x, r[2].y, r[2].z, r[2].w}, {r[3].x, r[3].y, r[3].z, r[3].w},
-                               {r[4].x, r[4].y, r[4].z, r[4].w}, {r[5].x, r[5].y, r[5].z, r[5].w},
-                               {r[6].x, r[6].y, r[6].z, r[6].w}, {r[7].x, r[7].y, r[7].z, r[7].w}};
-    uint4* base = reinterpret_cast<uint4*>(tile) + chunk_of(oct, ch);
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;  // high / low halves of a channel pair
-      uint4 o;
-      o.x = __builtin_amdgcn_perm(in[1][c >> 1], in[0][c >> 1], sel);
-      o.y = __builtin_amdgcn_perm(in[3][c >> 1], in[2][c >> 1], sel);
-      o.z = __builtin_amdgcn_perm(in[5][c >> 1], in[4][c >> 1], sel);
-      o.w = __builtin_amdgcn_perm(in[7][c >> 1], in[6][c >> 1], sel);
-      base[c] = o;
-    }
-  }
-};
-
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_big_kernel(
-    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
-    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint16_t* tiles = reinterpret_cast<uint16_t*>(smem);  // [stage][A,B][OP_ELEMS]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int L = xcd_remap(blockIdx.x, ntri * splits);
-  const int split = L / ntri;
-  int tm, tn;
-  blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
-  const int m0 = tm * T2, n0 = tn * T2;
-  const int tbeg = split * tokens_per_split;
-  const int tend = min(n, tbeg + tokens_per_split);
-
-  floatx16 acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  // patches of this thread: waves 0,1 stage the A tile, waves 2,3 the B tile; token octets oct and oct+4
-  const int opnd = wave >> 1;
-  const int co = lane & 31;                         // channel octet
-  const int oct = ((wave & 1) << 1) | (lane >> 5);  // 0..3
-  const int cbase = (opnd ? n0 : m0) + 8 * co;
-  Patch8 p0, p1;
-  const int nk = (tend - tbeg + KT2 - 1) / KT2;
-  const bool interior = (m0 + T2 <= C) && (n0 + T2 <= C);  // wave-uniform: no channel of the tile is out of range
-  if (nk > 0) {
-    p0.load<true>(X, ldx, tbeg + 8 * oct, tend, cbase, C);
-    p1.load<true>(X, ldx, tbeg + 8 * (oct + 4), tend, cbase, C);
-    p0.store(tiles + opnd * OP_ELEMS, 8 * co, oct);
-    p1.store(tiles + opnd * OP_ELEMS, 8 * co, oct + 4);
-  }
-  __syncthreads();
-  const int lr = lane & 31, lk = lane >> 5;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      const int t0 = tbeg + (kt + 1) * KT2;
-      if (interior && t0 + KT2 <= tend) {
-        p0.load<false>(X, ldx, t0 + 8 * oct, tend, cbase, C);
-        p1.load<false>(X, ldx, t0 + 8 * (oct + 4), tend, cbase, C);
-      } else {
-        p0.load<true>(X, ldx, t0 + 8 * oct, tend, cbase, C);
-        p1.load<true>(X, ldx, t0 + 8 * (oct + 4), tend, cbase, C);
-      }
-    }
-    const uint4* as = reinterpret_cast<const uint4*>(tiles + (cur * 2 + 0) * OP_ELEMS);
-    const uint4* bs = reinterpret_cast<const uint4*>(tiles + (cur * 2 + 1) * OP_ELEMS);
-    uint4 fa[2][4], fb[2][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      fa[0][i] = as[chunk_of(lk, wm * 128 + i * 32 + lr)];
-      fb[0][i] = bs[chunk_of(lk, wn * 128 + i * 32 + lr)];
-    }
-#pragma unroll
-    for (int kk = 0; kk < KT2 / 16; ++kk) {
-      if (kk + 1 < KT2 / 16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          fa[(kk + 1) & 1][i] = as[chunk_of(2 * (kk + 1) + lk, wm * 128 + i * 32 + lr)];
-          fb[(kk + 1) & 1][i] = bs[chunk_of(2 * (kk + 1) + lk, wn * 128 + i * 32 + lr)];
-        }
-      }
-      // keep the fragment reads of the next step ahead of this step's MFMAs (the scheduler would
-      // otherwise sink each read to just before its first use and expose the LDS latency)
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8n, fa[kk & 1][i]),
-                                                              __builtin_bit_cast(bf16x8n, fb[kk & 1][j]), acc[i][j], 0,
-                                                              0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (kt + 1 < nk) {
-      uint16_t* nx = tiles + ((cur ^ 1) * 2 + opnd) * OP_ELEMS;
-      p0.store(nx, 8 * co, oct);
-      p1.store(nx, 8 * co, oct + 4);
-    }
-    __syncthreads();
-  }
-
-  // epilogue straight from the accumulators: for a fixed register the 32 lanes of a half-wave cover
-  // 128 contiguous bytes of one row
-  const bool partial = splits > 1;
-  float* out = partial ? ws + ((long)split * ntri + (L - split * ntri)) * (T2 * T2) : H;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int c = wn * 128 + j * 32 + lr;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
-        if (partial) {
-          out[r * T2 + c] = acc[i][j][v];
-        } else if (m0 + r < C && n0 + c < C) {
-          float* q = H + (long)(m0 + r) * ldh + n0 + c;
-          float val = alpha * acc[i][j][v];
-          if (beta != 0.f) val = fmaf(beta, *q, val);
-          *q = val;
-        }
-      }
-    }
 }
 
 // =============================================================================================
@@ -476,31 +310,45 @@ __device__ __forceinline__ void dma_stage(const uint16_t* __restrict__ X, unsign
   }
 }
 
-// one 256x256 tile (or one token split of it); bid = linear workgroup index among ntri*splits.
+// How a call's tiles are dealt to workgroups.  The first `head` upper-triangle tiles (in blocked order) are computed
+// whole, one workgroup each, and written straight to H.  The remaining `ntail` tiles are cut into `splits` token
+// ranges of `tps` tokens, one workgroup per piece; the pieces go to the workspace as raw fp32 sums,
+// ws[(split * ntail + tail tile) * 256 * 256], and a second kernel adds them up in a fixed order.  Two uses: few
+// tiles in all (head = 0: the token ranges supply the parallelism), and the last, partly filled round of a large
+// triangle (406 tiles on 256 CUs: the 150 left over would keep the chip 59% busy for a whole round).
+struct SyrkPlan {
+  int ntri, head, ntail, splits, tps;
+};
+
+// one 256x256 tile (or one token range of it); (bid, yrow) = workgroup index in a grid of max(head, ntail) x (1 + splits),
+// or of head x 1 when nothing is cut.
 // NW = 4: four wavefronts of 128x128 (one per SIMD, all 512 registers).  NW = 8: eight of 128x64, two per SIMD:
 // while one waits for the address unit to take its direct loads the other keeps the matrix pipe busy.
 template <int NW, bool F16>
 __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx,
-                                              int n, int C, float alpha, float beta, int ntri, int splits,
-                                              int tokens_per_split, float* __restrict__ ws, int bid,
-                                              unsigned char* smem) {
+                                              int n, int C, float alpha, float beta, SyrkPlan pl, float* __restrict__ ws,
+                                              int bid, int yrow, unsigned char* smem) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // a scalar: LDS targets of the direct loads live in M0
   constexpr int NJ = 16 / NW;     // 32-column blocks per wavefront: 4 (128 columns) or 2 (64 columns)
   constexpr int WCOLS = NW / 2;   // wavefronts side by side along the columns
   constexpr int LPW = 32 / NW;    // direct loads per wavefront per stage
   const int wm = wave / WCOLS, wn = wave % WCOLS;
-  const int L = xcd_remap(bid, ntri * splits);
-  const int split = L / ntri;
+  // grid row 0: the whole tiles; grid row 1 + s: token range s of the tail tiles (pieces of one token range lie
+  // side by side: they share the rows of X they read).  Rows are as wide as the longer of the two: the rest leaves.
+  const int split = max(yrow - 1, 0);
+  const bool partial = yrow > 0;
+  if (bid >= (partial ? pl.ntail : pl.head)) return;
+  const int L = partial ? pl.head + bid : xcd_remap(bid, pl.head);
   int tm, tn;
-  blocked_tri_decode(L - split * ntri, (C + T2 - 1) / T2, tm, tn);
+  blocked_tri_decode(L, (C + T2 - 1) / T2, tm, tn);
   // uniform values that the division and the square root above left in vector registers: back to scalars,
   // the direct loads take their base address and LDS target from scalar registers
   tm = __builtin_amdgcn_readfirstlane(tm);
   tn = __builtin_amdgcn_readfirstlane(tn);
   const int m0 = tm * T2, n0 = tn * T2;
-  const int tbeg = __builtin_amdgcn_readfirstlane(split * tokens_per_split);
-  const int tend = min(n, tbeg + tokens_per_split);
+  const int tbeg = partial ? __builtin_amdgcn_readfirstlane(min(n, split * pl.tps)) : 0;
+  const int tend = partial ? min(n, tbeg + pl.tps) : n;
   const int nk = (tend - tbeg + KT3 - 1) / KT3;
   const bool interior = (m0 + T2 <= C) && (n0 + T2 <= C);
   // LDS byte address of the staging area plus this wavefront's share of a stage, as a scalar
@@ -582,8 +430,7 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
 #undef MQ_SYRK_ISSUE
 
   const int lr = lane & 31, lk = lane >> 5;
-  const bool partial = splits > 1;
-  float* out = partial ? ws + ((long)split * ntri + (L - split * ntri)) * (T2 * T2) : H;
+  float* out = partial ? ws + ((long)split * pl.ntail + (L - pl.head)) * (T2 * T2) : H;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -604,19 +451,12 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
     }
 }
 
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void syrk_bf16_dma_kernel(
-    float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
-    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
-  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  syrk_dma_tile<4, false>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
-}
-
 template <bool F16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_bf16_dma8_kernel(
     float* __restrict__ H, long ldh, const uint16_t* __restrict__ X, long ldx, int n, int C, float alpha, float beta,
-    int ntri, int splits, int tokens_per_split, float* __restrict__ ws) {
+    SyrkPlan pl, float* __restrict__ ws) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-  syrk_dma_tile<8, F16>(H, ldh, X, ldx, n, C, alpha, beta, ntri, splits, tokens_per_split, ws, blockIdx.x, smem);
+  syrk_dma_tile<8, F16>(H, ldh, X, ldx, n, C, alpha, beta, pl, ws, blockIdx.x, blockIdx.y, smem);
 }
 
 // Several independent accumulations (one Hessian each, same C) in one launch: blockIdx.y picks the problem.
@@ -635,23 +475,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     SyrkGroupTable t, int C, int ntri) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   const int z = blockIdx.y;
-  const int tps = (t.n[z] + KT3 - 1) / KT3 * KT3;
-  syrk_dma_tile<8, F16>(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], ntri, 1, tps, nullptr, blockIdx.x,
-                smem);
+  syrk_dma_tile<8, F16>(t.H[z], t.ldh[z], t.X[z], t.ldx[z], t.n[z], C, t.alpha[z], t.beta[z], SyrkPlan{ntri, ntri, 0, 1, 0},
+                        nullptr, blockIdx.x, 0, smem);
 }
 
-// fixed-order sum of the split partials of the big kernel; upper tiles only
+// fixed-order sum of the token-range pieces of the tail tiles (see SyrkPlan)
 __global__ __launch_bounds__(256) void syrk_big_reduce_kernel(float* __restrict__ H, long ldh, int C, float alpha,
-                                                              float beta, int ntri, int splits,
-                                                              const float* __restrict__ ws) {
-  const int L = blockIdx.y;
+                                                              float beta, SyrkPlan pl, const float* __restrict__ ws) {
+  const int lt = blockIdx.y;  // tail tile
   int tm, tn;
-  blocked_tri_decode(L, (C + T2 - 1) / T2, tm, tn);
+  blocked_tri_decode(pl.head + lt, (C + T2 - 1) / T2, tm, tn);
   const int idx = blockIdx.x * 256 + threadIdx.x;  // one float4 of the tile
   const int r = idx >> 6, c = (idx & 63) << 2;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int k = 0; k < splits; ++k) {
-    const float4 v = *reinterpret_cast<const float4*>(ws + ((long)k * ntri + L) * (T2 * T2) + r * T2 + c);
+  for (int k = 0; k < pl.splits; ++k) {
+    const float4 v = *reinterpret_cast<const float4*>(ws + ((long)k * pl.ntail + lt) * (T2 * T2) + r * T2 + c);
     s.x += v.x;
     s.y += v.y;
     s.z += v.z;
@@ -698,20 +536,48 @@ __global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, 
   }
 }
 
-void pick_split_big(int n, int C, int& ntri, int& splits, int& tps) {
+constexpr int NCU = 256;  // workgroups the large-tile kernel keeps resident (one per CU)
+
+SyrkPlan plan_big(int n, int C) {
   const int tiles = (C + T2 - 1) / T2;
-  ntri = tiles * (tiles + 1) / 2;
-  splits = 1;
-  if (ntri < 224) splits = (256 + ntri - 1) / ntri;  // one workgroup per CU is the most this kernel runs
-  const int max_splits = (n + 2047) / 2048;          // at least 2048 tokens per split
-  if (splits > max_splits) splits = max_splits;
-  if (splits > 64) splits = 64;
-  if (splits < 1) splits = 1;
-  tps = (n + splits - 1) / splits;
-  tps = (tps + KT2 - 1) / KT2 * KT2;
-  splits = (n + tps - 1) / tps;
-  if (splits < 1) splits = 1;
+  SyrkPlan pl;
+  pl.ntri = tiles * (tiles + 1) / 2;
+  pl.head = pl.ntri, pl.ntail = 0, pl.splits = 1, pl.tps = 0;
+  int splits = 1;
+  if (pl.ntri < 224) {  // too few tiles for the chip: every tile is cut, at least 2048 tokens per piece
+    splits = (NCU + pl.ntri - 1) / pl.ntri;
+    const int max_splits = (n + 2047) / 2048;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 64) splits = 64;
+    if (splits > 1) pl.head = 0;
+  } else {
+    // The last round holds rem = ntri % NCU tiles.  Cutting them into S pieces shortens that round from 1 to
+    // ceil(rem * S / NCU) / S tile times at the price of 256 KB written and read per piece, which pays when a
+    // tile time is long: from 32768 tokens on, at least 4096 tokens per piece.
+    static const bool tail_split = !(getenv("MQ_SYRK_TAIL") && atoi(getenv("MQ_SYRK_TAIL")) == 0);
+    const int rem = pl.ntri % NCU;
+    if (tail_split && rem > 0 && rem < 224 && n >= 32768) {
+      double best = 1.0;
+      for (int S = 2; S <= 8 && n / S >= 4096; ++S) {
+        const double cost = (double)((rem * S + NCU - 1) / NCU) / S;
+        if (cost < best - 0.04) best = cost, splits = S;
+      }
+      if (splits > 1) pl.head = pl.ntri - rem;
+    }
+  }
+  if (splits > 1) {
+    int tps = (n + splits - 1) / splits;
+    tps = (tps + KT3 - 1) / KT3 * KT3;
+    splits = (n + tps - 1) / tps;
+    if (splits > 1) {
+      pl.ntail = pl.ntri - pl.head, pl.splits = splits, pl.tps = tps;
+    } else {
+      pl.head = pl.ntri;
+    }
+  }
+  return pl;
 }
+size_t plan_big_ws_bytes(const SyrkPlan& pl) { return (size_t)pl.ntail * pl.splits * T2 * T2 * sizeof(float); }
 
 bool use_big(const void* X, long ldx, int n, int C) {
   return n >= 256 && C >= 256 && (C % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
@@ -741,8 +607,7 @@ extern "C" size_t mq_hessian_syrk_workspace_bytes(int n, int C) {
   int ntri, splits, tps;
   pick_split(n, C, ntri, splits, tps);
   const size_t small = splits > 1 ? (size_t)splits * ntri * T * T * sizeof(float) : 0;
-  pick_split_big(n, C, ntri, splits, tps);
-  const size_t big = splits > 1 ? (size_t)splits * ntri * T2 * T2 * sizeof(float) : 0;
+  const size_t big = plan_big_ws_bytes(plan_big(n, C));
   return small > big ? small : big;  // either kernel may be chosen, depending on alignment
 }
 
@@ -777,11 +642,7 @@ extern "C" int mq_hessian_syrk(float* H, long ldh, const void* X, int x_dtype, l
   if ((C & 1) || (ldx & 1) || ((uintptr_t)X & 3)) return MQ_ERR_ARG;  // 4-byte channel-pair loads
   int ntri, splits, tps;
   static std::once_flag once;
-  static bool use_dma = true;
-  static int dma_waves = 8;
   std::call_once(once, [] {
-    (void)hipFuncSetAttribute((const void*)syrk_bf16_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)BIG_SMEM);
-    (void)hipFuncSetAttribute((const void*)syrk_bf16_dma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)DMA_SMEM);
     (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)DMA_SMEM);
     (void)hipFuncSetAttribute((const void*)syrk_bf16_dma8_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -791,32 +652,23 @@ extern "C" int mq_hessian_syrk(float* H, long ldh, const void* X, int x_dtype, l
     (void)hipFuncSetAttribute((const void*)syrk_bf16_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)SMEM_BYTES);
     (void)hipFuncSetAttribute((const void*)syrk_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);
-    use_dma = getenv("MQ_SYRK_OLD") == nullptr;
-    dma_waves = getenv("MQ_SYRK_W4") ? 4 : 8;  // the one-wavefront-per-SIMD kernel stays for comparison (bf16 only)
   });
   if (n > 0 && use_big(X, ldx, n, C)) {
-    pick_split_big(n, C, ntri, splits, tps);
-    if (splits > 1) {
-      const size_t need = (size_t)splits * ntri * T2 * T2 * sizeof(float);
-      if (!workspace || workspace_bytes < need) return MQ_ERR_WORKSPACE;
-    }
+    const SyrkPlan pl = plan_big(n, C);
+    const size_t need = plan_big_ws_bytes(pl);
+    if (need && (!workspace || workspace_bytes < need)) return MQ_ERR_WORKSPACE;
+    const dim3 grid(pl.head > pl.ntail ? pl.head : pl.ntail, pl.ntail ? 1 + pl.splits : 1);
     if (f16)
-      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<true>, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh,
-                         (const uint16_t*)X, ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
-    else if (use_dma && dma_waves == 8)
-      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<false>, dim3(ntri * splits), dim3(512), DMA_SMEM, st, H, ldh,
-                         (const uint16_t*)X, ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
-    else if (use_dma)
-      hipLaunchKernelGGL(syrk_bf16_dma_kernel, dim3(ntri * splits), dim3(256), DMA_SMEM, st, H, ldh, (const uint16_t*)X,
-                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<true>, grid, dim3(512), DMA_SMEM, st, H, ldh, (const uint16_t*)X, ldx,
+                         n, C, alpha, beta, pl, (float*)workspace);
     else
-      hipLaunchKernelGGL(syrk_bf16_big_kernel, dim3(ntri * splits), dim3(256), BIG_SMEM, st, H, ldh, (const uint16_t*)X,
-                         ldx, n, C, alpha, beta, ntri, splits, tps, (float*)workspace);
+      hipLaunchKernelGGL(syrk_bf16_dma8_kernel<false>, grid, dim3(512), DMA_SMEM, st, H, ldh, (const uint16_t*)X, ldx,
+                         n, C, alpha, beta, pl, (float*)workspace);
     int rc = mq_check_launch();
     if (rc != MQ_OK) return rc;
-    if (splits > 1) {
-      hipLaunchKernelGGL(syrk_big_reduce_kernel, dim3(T2 * T2 / 4 / 256, ntri), dim3(256), 0, st, H, ldh, C, alpha, beta,
-                         ntri, splits, (const float*)workspace);
+    if (pl.ntail) {
+      hipLaunchKernelGGL(syrk_big_reduce_kernel, dim3(T2 * T2 / 4 / 256, pl.ntail), dim3(256), 0, st, H, ldh, C, alpha, beta,
+                         pl, (const float*)workspace);
       if ((rc = mq_check_launch()) != MQ_OK) return rc;
     }
     return mirror ? mq_symmetrize_upper(H, ldh, C, stream) : MQ_OK;

@@ -277,7 +277,7 @@ class GPTQ:
             perm_i32, perm_inv_i32 = perm.to(torch.int32), perm_inv.to(torch.int32)
             self._perm = perm
             if tied is None:
-                self.H = self.H[perm][:, perm]
+                self.H = ops.permute_symmetric(self.H, perm_i32)  # src/gptq.py:187, one pass, no second temporary
         if perm is None:
             scale_row = torch.arange(d_col, device=device, dtype=torch.int32) // group_size
         else:

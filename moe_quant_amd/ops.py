@@ -138,6 +138,21 @@ def hessian_prestep_(H: Tensor, upper_only: bool) -> Tuple[Tensor, Tensor]:
     return pruned, flags
 
 
+def permute_symmetric(H: Tensor, perm: Tensor) -> Tensor:
+    """H[perm][:, perm] as a new tensor, in one pass (perm: int32 of length C on the device)."""
+    _dev(H, perm)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride")
+    if perm.dtype != torch.int32 or perm.numel() != C or not perm.is_contiguous():
+        raise ValueError("perm must be a contiguous int32 vector of length C")
+    Hp = torch.empty((C, C), dtype=torch.float32, device=H.device)
+    check(lib.mq_permute_symmetric(H.data_ptr(), H.stride(0), perm.data_ptr(), Hp.data_ptr(), C, C, _stream(H)),
+          "mq_permute_symmetric")
+    return Hp
+
+
 def hessian_damp_(H: Tensor, W: Tensor, pruned: Optional[Tensor], rel_damp: float, flags: Tensor) -> Tensor:
     """In place: rows/columns of H for all-zero (or pruned) weight columns cleared with a unit diagonal, then
     rel_damp * mean(diag) added to the diagonal."""

@@ -733,3 +733,42 @@ def test_loop_chol_matches_classical_loop(dev, C, R, order):
                                      [o[4] for o in outs], 8.0, 15.0, torch.bfloat16, 128)
     for i in range(3):
         assert torch.equal(Qg[i], outs[i][1]) and torch.equal(pairs[i][0], outs[i][0])
+
+
+@pytest.mark.parametrize("C", [128, 1000, 7168, 18432])
+def test_permute_symmetric_equals_torch_gather(dev, C):
+    """Act-order gather (src/gptq.py:187): bit-identical to H[perm][:, perm], input untouched."""
+    g = torch.Generator(device=dev).manual_seed(C)
+    H = torch.randn(C, C, generator=g, device=dev)
+    perm = torch.argsort(H.diag(), descending=True)
+    keep = H.clone() if C <= 7168 else None
+    Hp = ops.permute_symmetric(H, perm.to(torch.int32))
+    assert torch.equal(Hp, H[perm][:, perm])
+    if keep is not None:
+        assert torch.equal(H, keep)
+
+
+def test_hessian_syrk_tail_round_split(dev):
+    """7168 channels are 406 tiles of 256x256 on 256 CUs: from 32768 tokens on the 150 tiles of the last round are cut
+    into token ranges whose partial sums meet in the workspace.  Against an fp64 product formed on the GPU, with a
+    ragged token count, accumulating onto an old H."""
+    from moe_quant_amd import _lib
+
+    C, n = 7168, 32768 + 40
+    assert _lib.load().mq_hessian_syrk_workspace_bytes(n, C) > 0 and _lib.load().mq_hessian_syrk_workspace_bytes(8192, C) == 0
+    g = torch.Generator(device=dev).manual_seed(5)
+    X = torch.randn(n, C, generator=g, device=dev)
+    X[:, synth.outlier_channels(C, 6).to(dev)] *= 20.0
+    X = X.to(torch.bfloat16)
+    H0 = torch.randn(C, C, generator=g, device=dev)
+    H0 = H0 + H0.t()
+    H = H0.clone()
+    ops.hessian_syrk_(H, X, 0.5, 2.0 / n, mirror=True)
+    ref = torch.zeros(C, C, device=dev, dtype=torch.float64)
+    for s0 in range(0, n, 8192):
+        blk = X[s0:s0 + 8192].double()
+        ref.addmm_(blk.t(), blk)
+    ref = 0.5 * H0.double() + (2.0 / n) * ref
+    err = ((H.double() - ref).norm() / ref.norm()).item()
+    _say(f"tail-split syrk rel err {err:.2e}")
+    assert err < 1e-5 and torch.equal(H, H.t())
