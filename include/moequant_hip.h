@@ -209,9 +209,11 @@ int mq_prepare_wt_pair(const void* W, int w_dtype, long ldw, int R, int C, const
  *   qzero : nullable, same indexing; NULL means the constant qzero_const.
  *   round_dtype : rounding of the dequantized value ((q - z) * s), the `dtype` of tl_dequantize.
  *   block : columns per lazy-batch block; values <= 0 or > 128 use 128 (only reassociates fp32 sums).
- *   Qt    : C x R u8 out, integer codes.   E : 8 x 128 x R fp32 scratch (a ring of error blocks: a block's
- *           sequential walk overlaps the trailing update of a batch of up to four blocks before it).
+ *   Qt    : C x R u8 out, integer codes.   E : mq_gptq_loop_scratch_bytes(R) bytes of scratch (a ring of sixteen
+ *           128 x R fp32 error blocks: a block's sequential walk overlaps the trailing update of a batch of up to
+ *           eight blocks before it).
  */
+size_t mq_gptq_loop_scratch_bytes(int R);
 int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale, long ld_scale,
                  const int* scale_row, const float* qzero, float qzero_const, float maxq, int round_dtype, int block,
                  uint8_t* Qt, float* E, void* stream);
@@ -272,6 +274,14 @@ int mq_gemm_f32(const float* A, long sam, long sak, const float* B, long sbk, lo
  */
 int mq_dequant_fp8_block(const uint8_t* W, long ldw, int R, int C, const float* scale_inv, long ld_scale, int out_dtype,
                          void* out, long ldo, void* stream);
+
+/* ---- the step before GPTQ.update of a down projection: the expert's SwiGLU product ------------------------------
+ * Replaces the elementwise part of the expert forward that feeds the down projection's hook (quant.py:280-281 runs the
+ * block; an expert computes act_fn(gate_proj(x)) * up_proj(x)): out[r, j] = round(round(silu(GU[r, j])) * GU[r, I + j])
+ * for GU (n x 2I, ldg) holding the gate projection's outputs followed by the up projection's (one GEMM against the
+ * stacked weights), both roundings to `dtype` (MQ_DT_BF16 / MQ_DT_F16) as the chained torch ops round.
+ *   I % 8 == 0, 16-byte aligned rows; out : n x I (ldo). */
+int mq_swiglu(const void* GU, long ldg, int n, int I, int dtype, void* out, long ldo, void* stream);
 
 #ifdef __cplusplus
 }

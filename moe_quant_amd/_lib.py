@@ -39,12 +39,14 @@ SIGNATURES = {
     "mq_prepare_wt_pair": (_i, [_vp, _i, _l, _i, _i, _vp, _vp, _vp, _vp, _l, _vp]),
     "mq_gptq_loop_chol": (_i, [_vp, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
     "mq_gptq_loop_chol_grouped": (_i, [_i, _vp, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
+    "mq_gptq_loop_scratch_bytes": (_sz, [_i]),
     "mq_gptq_loop": (_i, [_vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
     "mq_gptq_loop_grouped": (_i, [_i, _vp, _l, _i, _i, _vp, _l, _vp, _l, _vp, _vp, _f, _f, _i, _i, _vp, _vp, _vp]),
     "mq_untranspose_codes": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
     "mq_pack_int4": (_i, [_vp, _l, _i, _i, _vp, _i, _vp, _l, _vp]),
     "mq_pack_from_qt": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
     "mq_dequant_fp8_block": (_i, [_vp, _l, _i, _i, _vp, _l, _i, _vp, _l, _vp]),
+    "mq_swiglu": (_i, [_vp, _l, _i, _i, _i, _vp, _l, _vp]),
     "mq_gemm_f32": (_i, [_vp, _l, _l, _vp, _l, _l, _vp, _l, _i, _i, _i, _f, _f, _i, _i, _vp]),
 }
 

@@ -32,7 +32,7 @@ constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
 constexpr int LDM = 132;   // LDS row pitch: rows 16-byte aligned, consecutive rows 4 banks apart (8 rows span the 32 banks)
 constexpr int SOFF = 4;    // column shift of the S triangle inside a row (keeps both triangles 16-byte aligned)
-static int TRAIL_PANELS = 4;  // panels per trailing update of the whole matrix (env MQ_PANELS)
+static int TRAIL_PANELS = 8;  // panels per trailing update of the whole matrix (env MQ_PANELS)
 static int INV_KC = 4;  // the first inverse product is cut into K chunks of 4 blocks (512), one workgroup each
 
 // ---------------------------------------------------------------------------------------------

@@ -32,9 +32,9 @@
 namespace {
 
 constexpr int B = 128;
-constexpr int LOOP_BATCH_MAX = 4;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
-static int LOOP_BATCH = 2;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..4;
-                                    // 1, 2, 3, 4: 300, 312, 312, 309 linears/s at four streams)
+constexpr int LOOP_BATCH_MAX = 8;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
+static int LOOP_BATCH = 4;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..8;
+                                    // 1, 2, 3, 4: 0.99, 0.83, 0.77, 0.75 ms per 2048x7168 linear in grouped calls of eight)
 
 __device__ __forceinline__ float round_dtype(float x, int rd) {
   // branch-free so that the unrolled column steps stay one basic block
@@ -242,6 +242,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   a.E = grp.E[e] + off.e_cur;
   a.Eprev = off.e_prev >= 0 ? grp.E[e] + off.e_prev : nullptr;
   if (bid >= ncol) {  // a tile of the trailing update due at this block
+    // (tiles in plain row-major order: the round-robin of workgroups over the eight XCDs then gives each XCD two
+    // of the sixteen column tiles of every row tile -- measured better, in time and in bytes fetched, than one
+    // contiguous run of tiles per XCD, whose working set of error blocks overflows the L2)
     const int idx = (bid - ncol) % tiles;
     g.A = a.U + off.g_a;
     g.B = grp.E[e] + off.g_b;
@@ -599,6 +602,10 @@ int loop_impl(int G, float* const* Wt, long ldw, int C, int R, const float* cons
 }
 
 }  // namespace
+
+extern "C" size_t mq_gptq_loop_scratch_bytes(int R) {
+  return R > 0 ? (size_t)2 * LOOP_BATCH_MAX * B * R * sizeof(float) : 0;
+}
 
 extern "C" int mq_gptq_loop(float* Wt, long ldw, int C, int R, const float* U, long ldu, const float* scale,
                             long ld_scale, const int* scale_row, const float* qzero, float qzero_const, float maxq,

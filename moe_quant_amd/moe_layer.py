@@ -17,6 +17,7 @@ from typing import Dict, List, Optional
 import torch
 import torch.nn as nn
 
+from . import ops
 from .gptq import GPTQ
 
 
@@ -103,11 +104,16 @@ def quantize_moe_layer(
     for e, (g, u, d) in enumerate(handles):
         lo, hi = offsets[e], offsets[e + 1]
         res.tokens_per_expert.append(hi - lo)
+        gate_up = None
         for s in range(lo, hi, max_rows_per_update):
             idx = rows[s : min(hi, s + max_rows_per_update)]
             xe = x.index_select(0, idx)  # (n, C) bf16
             g.update(xe)
-            a = torch.nn.functional.silu(xe @ experts[e].gate.t()) * (xe @ experts[e].up.t())  # the expert's forward
+            # the expert's forward up to the down projection's input: one GEMM against the stacked gate/up weights
+            # (the model's own matmul, rocBLAS/hipBLASLt through torch), then the SwiGLU product in one pass
+            if gate_up is None:
+                gate_up = torch.cat([experts[e].gate, experts[e].up], dim=0)
+            a = ops.swiglu(xe @ gate_up.t())
             d.update(a)
             if e in keep_codes:
                 prev = res.down_inputs.get(e)

@@ -378,7 +378,7 @@ def gptq_loop_chol_grouped_(Wts, W0ts, Fs, scales, scale_rows, qzero_const: floa
         raise ValueError("scale must be (C,R) when no scale_row map is given")
     dev = Wts[0].device
     Qts = [torch.empty(C, R, dtype=torch.uint8, device=dev) for _ in range(k)]
-    ring = 8 * 128 * R * 4
+    ring = lib.mq_gptq_loop_scratch_bytes(R)
     E = _ws.get(dev, ring * k, "loop")
     import ctypes as C_
 
@@ -406,7 +406,7 @@ def gptq_loop_(Wt: Tensor, U: Tensor, scale: Tensor, scale_row: Optional[Tensor]
     if scale_row is None and scale.shape[0] != C:
         raise ValueError("scale must be (C,R) when no scale_row map is given")
     Qt = torch.empty(C, R, dtype=torch.uint8, device=Wt.device)
-    E = _ws.get(Wt.device, 8 * 128 * R * 4, "loop")
+    E = _ws.get(Wt.device, lib.mq_gptq_loop_scratch_bytes(R), "loop")
     rc = lib.mq_gptq_loop(Wt.data_ptr(), Wt.stride(0), C, R, U.data_ptr(), U.stride(0), scale.data_ptr(),
                           scale.stride(0), _p(scale_row), _p(qzero), qzero_const, maxq, _dt(round_dtype), block,
                           Qt.data_ptr(), E.data_ptr(), _stream(Wt))
@@ -440,7 +440,7 @@ def gptq_loop_grouped_(Wts, Us, scales, scale_rows, qzero_const: float, maxq: fl
         raise ValueError("scale must be (C,R) when no scale_row map is given")
     dev = Wts[0].device
     Qts = [torch.empty(C, R, dtype=torch.uint8, device=dev) for _ in range(k)]
-    ring = 8 * 128 * R * 4
+    ring = lib.mq_gptq_loop_scratch_bytes(R)
     E = _ws.get(dev, ring * k, "loop")
     import ctypes as C_
 
@@ -511,6 +511,18 @@ def dequant_fp8_block(W: Tensor, scale_inv: Tensor, dtype: torch.dtype) -> Tenso
     rc = lib.mq_dequant_fp8_block(W.data_ptr(), W.stride(0), R, C, s.data_ptr(), s.stride(0), _dt(dtype), out.data_ptr(),
                                   out.stride(0), _stream(W))
     check(rc, "mq_dequant_fp8_block")
+    return out
+
+
+def swiglu(GU: Tensor) -> Tensor:
+    """silu(GU[:, :I]) * GU[:, I:] for a (n, 2I) bf16/fp16 matrix of gate outputs followed by up outputs."""
+    _dev(GU)
+    lib = _lib.load()
+    if GU.dim() != 2 or GU.dtype not in (torch.bfloat16, torch.float16) or GU.shape[1] % 16 or GU.stride(1) != 1:
+        raise ValueError("GU must be (n, 2I) bf16/fp16 with unit column stride and I % 8 == 0")
+    n, I = GU.shape[0], GU.shape[1] // 2
+    out = torch.empty(n, I, dtype=GU.dtype, device=GU.device)
+    check(lib.mq_swiglu(GU.data_ptr(), GU.stride(0), n, I, _dt(GU.dtype), out.data_ptr(), I, _stream(GU)), "mq_swiglu")
     return out
 
 

@@ -772,3 +772,19 @@ def test_hessian_syrk_tail_round_split(dev):
     err = ((H.double() - ref).norm() / ref.norm()).item()
     _say(f"tail-split syrk rel err {err:.2e}")
     assert err < 1e-5 and torch.equal(H, H.t())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,I", [(1, 8), (37, 2048), (700, 512), (0, 64)])
+def test_swiglu_against_the_torch_expression(dev, n, I, dtype):
+    """silu(g) * u as the chained torch ops compute it on 16-bit tensors (each op rounds its result): equal up to one
+    unit in the last place of the 16-bit result (the exponential inside silu differs in its last fp32 bits)."""
+    g = torch.Generator(device=dev).manual_seed(n + I)
+    GU = (torch.randn(n, 2 * I, generator=g, device=dev) * 3).to(dtype)
+    got = ops.swiglu(GU)
+    want = torch.nn.functional.silu(GU[:, :I]) * GU[:, I:]
+    assert got.shape == want.shape and got.dtype == dtype
+    if n:
+        ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+        assert ((got.float() - want.float()).abs() <= ulp * want.float().abs() + 1e-30).all()
+        assert (got == want).float().mean().item() > 0.99
