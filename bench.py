@@ -34,8 +34,9 @@ def parse():
                     help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
-    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer"],
-                    help="config1 (default, the benchmark line) or moe_layer (config 3: whole MoE layer, one pass)")
+    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer", "gemm"],
+                    help="config1 (default, the benchmark line), moe_layer (config 3: whole MoE layer, one pass) or gemm "
+                         "(micro-benchmark of the fp32 GEMM core shared by the factorisation and the loop)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--tokens", type=int, default=2_097_152)
     ap.add_argument("--check-experts", type=int, default=2, help="moe_layer: experts compared with the CPU oracle")
@@ -46,8 +47,8 @@ def parse():
 
 def traffic_from_profiles(call, **keys):
     """HBM bytes per call of `call` for the configuration `keys`, from the table of measured traffic committed in
-    profiles/hbm_traffic.md (lines of the form `| call | C=7168 G=8 panels=4 | 1.23e9 | ...`); None if absent."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+    profiles/config1_bench_hbm_traffic.md (lines of the form `| call | C=7168 G=8 panels=8 | 2.4e10 | ...`); None if absent."""
+    path = os.path.join(ROOT, "profiles", "config1_bench_hbm_traffic.md")
     if not os.path.exists(path):
         return None
     want = " ".join(f"{k}={v}" for k, v in keys.items())
@@ -151,6 +152,41 @@ def moe_layer_main(args):
     print(json.dumps(out))
 
 
+def gemm_main(args):
+    """Micro-benchmark of mq_gemm_f32 (fp32 in and out; interior tiles form each product from six bf16-piece products
+    on the bf16 matrix cores): the shapes the factorisation and the loop issue.  One JSON line, TFLOP/s per shape."""
+    import torch
+
+    from moe_quant_amd import _lib, ops
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    shapes = [(4096, 4096, 4096, 0.0), (8192, 8192, 128, 1.0), (8192, 8192, 256, 1.0), (8192, 8192, 512, 1.0),
+              (8192, 8192, 1024, 1.0), (7040, 2048, 128, 1.0), (6656, 2048, 512, 1.0)]
+    out = {}
+    for M, N, K, beta in shapes:
+        A = torch.randn(M, K, generator=g, device=dev)
+        Bm = torch.randn(N, K, generator=g, device=dev)  # B(k,n) = Bm[n,k]: both operands K-contiguous
+        Cm = torch.zeros(M, N, device=dev)
+        run = lambda: ops.gemm_f32_(A, K, 1, Bm, 1, K, Cm, M, N, K, alpha=1.0, beta=beta)
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 20
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[f"{M}x{N}x{K} beta={beta:g}"] = {"ms": round(ms, 4), "tflops": round(2.0 * M * N * K / ms / 1e9, 1)}
+    print(json.dumps({"metric": "fp32 GEMM core TFLOP/s (fp32 in/out, six bf16-piece products per fp32 product)",
+                      "unit": "TFLOP/s", "n_gpus": 1, "dtype": "f32", "data": "synthetic", "peak_fp32_mfma": PEAK_FP32_MFMA,
+                      "shapes": out}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -158,6 +194,8 @@ def main():
         sys.exit(2)
     if args.workload == "moe_layer":
         return moe_layer_main(args)
+    if args.workload == "gemm":
+        return gemm_main(args)
     import torch
 
     from moe_quant_amd import _lib, ops, synth
@@ -320,7 +358,7 @@ def main():
     # above with HIP events on the launch stream.  traffic = HBM bytes per call from the rocprofv3 --pmc runs
     # summarised in profiles/ (looked up by matrix size, group size and panel batch; null when that table has no
     # line for this configuration).
-    panels = int(os.environ.get("MQ_PANELS", "4") or 4)
+    panels = int(os.environ.get("MQ_PANELS", "8") or 8)
     traffic = traffic_from_profiles("mq_factor_chol_grouped", C=C, G=Gq, panels=panels)
     roofline = {
         "kernel": f"mq_factor_chol_grouped over {Gq} matrices = trail_diag_kernel + panel_inv_kernel + revchol_diag_kernel + "

@@ -180,6 +180,16 @@ def pack_checkpoint(model_name_or_path: str, quantized_model_path: str, packed_m
         m = re.match(r"model\.layers\.(\d+)\.", k)
         (block_keys[int(m.group(1))] if m else rest).append(k)
     n_blocks = max(block_keys) + 1 if block_keys else 0
+    cfg_path = os.path.join(model_name_or_path, "config.json")
+    cfg = {}
+    if os.path.exists(cfg_path):
+        with open(cfg_path) as f:
+            cfg = json.load(f)
+    # The reference walks the blocks of the model built from config.json (pack_quantized_model.py:140-186): tensors
+    # of layers beyond num_hidden_layers (DeepSeek-V3's multi-token-prediction layer 61) belong to no block of that
+    # model and are not written.
+    if isinstance(cfg.get("num_hidden_layers"), int):
+        n_blocks = min(n_blocks, cfg["num_hidden_layers"])
     num_output_shards = n_blocks + 2
     quantized = quantized_layers_by_block(quantized_model_path)
     index: Dict[str, str] = {}
@@ -201,11 +211,6 @@ def pack_checkpoint(model_name_or_path: str, quantized_model_path: str, packed_m
     last = [k for k in rest if k not in first]
     save_packed_shard(dequantized(shards.load(last)), packed_model_path, num_output_shards, num_output_shards, index)
     save_safetensors_index(packed_model_path, index)
-    cfg_path = os.path.join(model_name_or_path, "config.json")
-    cfg = {}
-    if os.path.exists(cfg_path):
-        with open(cfg_path) as f:
-            cfg = json.load(f)
     cfg.pop("quantization_config", None)  # the source's FP8 description no longer applies (pack_quantized_model.py:118-119)
     cfg["quantization_config"] = prepare_quantization_config(bits, group_size, only_experts)
     with open(os.path.join(packed_model_path, "config.json"), "w") as f:

@@ -186,6 +186,8 @@ def test_pack_command_line_on_a_synthetic_checkpoint(dev, tmp_path):
             name = f"{pre}mlp.experts.0.{proj}"
             tensors[name + ".weight"] = (torch.randn(R, C, generator=g) * 0.02).bfloat16()
             qnames.append(name)
+    # a layer beyond num_hidden_layers (DeepSeek-V3 ships its multi-token-prediction layer that way): not packed
+    tensors["model.layers.2.embed_tokens.weight"] = torch.randn(50, 64, generator=g).bfloat16()
     fp8_name = "model.layers.1.self_attn.o_proj"
     w8 = (torch.randn(R, C, generator=g) * 0.5).to(torch.float8_e4m3fn)
     s8 = torch.rand(R // 128, C // 128, generator=g) * 0.1 + 0.01
@@ -198,7 +200,8 @@ def test_pack_command_line_on_a_synthetic_checkpoint(dev, tmp_path):
         save_file({k: tensors[k].contiguous() for k in ks}, str(src / fn))
         wm.update({k: fn for k in ks})
     json.dump({"metadata": {}, "weight_map": wm}, open(src / "model.safetensors.index.json", "w"))
-    json.dump({"hidden_size": 64, "quantization_config": {"quant_method": "fp8"}}, open(src / "config.json", "w"))
+    json.dump({"hidden_size": 64, "num_hidden_layers": 2, "quantization_config": {"quant_method": "fp8"}},
+              open(src / "config.json", "w"))
     (src / "tokenizer.json").write_text("{}")
     blobs = {}
     for name in qnames:
@@ -217,7 +220,7 @@ def test_pack_command_line_on_a_synthetic_checkpoint(dev, tmp_path):
     back = {}
     for fn in shards:
         back.update(load_file(str(pdir / fn)))
-    assert set(back) == set(out_wm)
+    assert set(back) == set(out_wm) and not any(k.startswith("model.layers.2.") for k in back)
     assert out_wm["model.embed_tokens.weight"] == shards[0] and out_wm["lm_head.weight"] == shards[3]
     assert out_wm["model.norm.weight"] == shards[3] and out_wm["model.layers.0.input_layernorm.weight"] == shards[1]
     for name in qnames:
