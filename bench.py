@@ -34,9 +34,10 @@ def parse():
                     help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
-    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer", "gemm"],
+    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer", "gemm", "syrk"],
                     help="config1 (default, the benchmark line), moe_layer (config 3: whole MoE layer, one pass) or gemm "
-                         "(micro-benchmark of the fp32 GEMM core shared by the factorisation and the loop)")
+                         "(micro-benchmark of the fp32 GEMM core shared by the factorisation and the loop) or syrk (the "
+                         "Hessian kernel beside the vendor library's GEMM on the same operands)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--tokens", type=int, default=2_097_152)
     ap.add_argument("--check-experts", type=int, default=2, help="moe_layer: experts compared with the CPU oracle")
@@ -187,6 +188,51 @@ def gemm_main(args):
                       "shapes": out}))
 
 
+def syrk_main(args):
+    """The Hessian kernel (upper triangle only, tokens read as the hooks deliver them: token-major) beside the vendor
+    GEMM torch dispatches for X^T X on the same tensor (full product), and beside the same GEMM on a pre-transposed
+    copy (both operands contiguous along the tokens, the layout matrix cores like best).  One JSON line."""
+    import torch
+
+    from moe_quant_amd import _lib, ops
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+
+    def timed(fn, reps=8):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    out = {}
+    for n, C in ((8192, 7168), (32768, 7168), (131072, 7168), (65536, 2048)):
+        X = torch.randn(n, C, device=dev).to(torch.bfloat16)
+        H = torch.zeros(C, C, device=dev)
+        alg = n * C * (C + 1)
+        t_own = timed(lambda: ops.hessian_syrk_(H, X, 0.0, 2.0 / n, mirror=False))
+        t_lib = timed(lambda: X.t() @ X)
+        Xt = X.t().contiguous()
+        t_lib_t = timed(lambda: Xt @ Xt.t())
+        out[f"n={n} C={C}"] = {
+            "mq_hessian_syrk_ms": round(t_own, 4), "algorithmic_tflops": round(alg / t_own / 1e9, 1),
+            "frac_bf16_peak": round(alg / t_own / 1e9 / PEAK_BF16_MFMA, 4),
+            "vendor_gemm_same_layout_ms": round(t_lib, 4),
+            "vendor_gemm_same_layout_executed_tflops": round(2.0 * n * C * C / t_lib / 1e9, 1),
+            "vendor_gemm_pretransposed_ms": round(t_lib_t, 4),
+            "vendor_gemm_pretransposed_executed_tflops": round(2.0 * n * C * C / t_lib_t / 1e9, 1),
+        }
+        del X, Xt, H
+    print(json.dumps({"metric": "Hessian SYRK TFLOP/s (algorithmic n*C*(C+1)) beside the vendor GEMM on the same operands",
+                      "unit": "TFLOP/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "peak_bf16_mfma": PEAK_BF16_MFMA,
+                      "shapes": out}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -196,6 +242,8 @@ def main():
         return moe_layer_main(args)
     if args.workload == "gemm":
         return gemm_main(args)
+    if args.workload == "syrk":
+        return syrk_main(args)
     import torch
 
     from moe_quant_amd import _lib, ops, synth
