@@ -91,13 +91,16 @@ def moe_layer_run(args, with_cpu_oracle=True):
     out = {
         "wall_s": round(res.seconds["total"], 3),
         "seconds": {k: round(v, 3) for k, v in res.seconds.items()},
+        "quantization_overlaps_hessian_collection": res.overlapped,
         "experts": args.experts, "tokens": args.tokens, "top_k": int(ids.shape[1]), "hidden": C, "inter": I,
         "linears": 3 * args.experts,
         "generate_inputs_s": round(t_gen, 2),
         "tokens_per_expert": {"min": int(n_e.min()), "max": int(n_e.max()), "mean": float(n_e.mean())},
         "hessian_algorithmic_tflop": round(flop_syrk / 1e12, 1),
         "issues": res.issues,
-        "note": "seconds.hessians counts the expert forward (gate/up products + SiLU product) that produces the "
+        "note": "seconds.hessians_... is the time of the Hessian stream (token gather, expert forward, SYRK) with the "
+                "quantization of earlier experts running beside it, seconds.quantize_and_pack the rest of the wall; "
+                "seconds.hessians counts the expert forward (gate/up products + SiLU product) that produces the "
                 "down-projection inputs; the model forward is not part of the GPTQ kernels' rooflines",
     }
     if check and with_cpu_oracle:

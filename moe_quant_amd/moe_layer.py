@@ -40,6 +40,7 @@ class LayerResult:
     issues: Dict[str, int] = field(default_factory=dict)
     issues_by_linear: Dict[str, List[str]] = field(default_factory=dict)  # "<e>.<proj>" -> names of raised flags
     factorizations: int = 0  # Hessian factorisations actually computed (a tied up_proj reuses its gate_proj's)
+    overlapped: bool = False  # quantization ran beside the collection of later Hessians (seconds then overlap too)
 
 
 def route_tokens(expert_ids: torch.Tensor, n_experts: int):
@@ -66,6 +67,7 @@ def quantize_moe_layer(
     max_rows_per_update: int = 1 << 17,
     streams: int = 2,
     group: int = 8,
+    overlap: bool = True,
 ) -> LayerResult:
     """x (T, C) bf16 on the GPU, expert_ids (T, top_k) int64 on the GPU.
 
@@ -74,7 +76,9 @@ def quantize_moe_layer(
     time -- their factorisations and column loops run as grouped library calls, every launch carrying the work of
     all of them -- and the groups go round-robin onto `streams` HIP streams, so that the short per-linear kernels
     of one group overlap the long launches of another.  Nothing in the path reads a value back to the host, so one
-    host thread keeps all streams fed."""
+    host thread keeps all streams fed.
+    `overlap`: quantize a group as soon as its Hessians are complete, beside the collection of the next group's
+    (False: the reference's order, every Hessian of the block first)."""
     dev = x.device
     E = len(experts)
     keep_codes = set(keep_codes or [])
@@ -93,17 +97,24 @@ def quantize_moe_layer(
         d = GPTQ(linear(ew.down), group_size, True, rel_damp, block_size)
         handles.append((g, u, d))
 
-    # ---- phase 1: Hessians of the whole block
     sync()
     t0 = time.perf_counter()
     rows, offsets = route_tokens(expert_ids, E)
     sync()
     res.seconds["route"] = time.perf_counter() - t0
-    t_gather = t_fwd = 0.0
-    t1 = time.perf_counter()
-    for e, (g, u, d) in enumerate(handles):
+    res.tokens_per_expert = [offsets[e + 1] - offsets[e] for e in range(E)]
+    main = torch.cuda.current_stream(dev)
+    n_lanes = max(1, streams)
+    # without overlap the current stream is lane 0; with overlap the Hessians keep the current stream to themselves
+    lanes = ([] if overlap else [main]) + [torch.cuda.Stream(device=dev) for _ in range(n_lanes - (0 if overlap else 1))]
+    done = []  # (name, handle): verdict words are read after everything is queued
+    factor_calls_before = GPTQ.factor_calls
+    group = max(1, group)
+
+    def collect_hessians(e):
+        """Hessians of expert e (gate and up share one, quant.py:258-277) from its routed tokens."""
+        g, u, d = handles[e]
         lo, hi = offsets[e], offsets[e + 1]
-        res.tokens_per_expert.append(hi - lo)
         gate_up = None
         for s in range(lo, hi, max_rows_per_update):
             idx = rows[s : min(hi, s + max_rows_per_update)]
@@ -118,58 +129,82 @@ def quantize_moe_layer(
             if e in keep_codes:
                 prev = res.down_inputs.get(e)
                 res.down_inputs[e] = a if prev is None else torch.cat([prev, a])
-    sync()
-    res.seconds["hessians_incl_gather_and_forward"] = time.perf_counter() - t1
 
-    # ---- phase 2: quantize + pack 3 linears per expert, experts round-robin over the streams
-    t2 = time.perf_counter()
-    main = torch.cuda.current_stream(dev)
-    lanes = [main] + [torch.cuda.Stream(device=dev) for _ in range(max(1, streams) - 1)]  # the current stream is lane 0
-    for s_ in lanes:
-        if s_ is not main:
-            s_.wait_stream(main)
-    done = []  # (name, handle): verdict words are read after everything is queued
-    factor_calls_before = GPTQ.factor_calls
-    group = max(1, group)
-    for ci, e0 in enumerate(range(0, E, group)):
-        chunk = list(range(e0, min(E, e0 + group)))
-        lane = lanes[ci % len(lanes)]
-        with torch.cuda.stream(lane):
+    def quantize_chunk(chunk):
+        """Quantize + pack the three linears of every expert of the chunk (on the current stream)."""
+        for e in chunk:
+            g, u, d = handles[e]
+            if e in keep_codes:
+                g.symmetrize_hessian()
+                d.symmetrize_hessian()
+                if g.H is not None:
+                    res.hessians[f"{e}.gate_proj"] = g.H.clone()
+                if d.H is not None:
+                    res.hessians[f"{e}.down_proj"] = d.H.clone()
+        # gate and up projections of the chunk (one factor per expert, shared), then the down projections
+        gu = [handles[e][i] for e in chunk for i in (0, 1)]
+        names = [(e, n) for e in chunk for n in ("gate_proj", "up_proj")] + [(e, "down_proj") for e in chunk]
+        dn = [handles[e][2] for e in chunk]
+        if group > 1:
+            outs = GPTQ.quantize_many(gu, bits) + GPTQ.quantize_many(dn, bits)
+        else:
+            outs = [h.quantize(bits) for h in gu + dn]
+        for (e, name), h, (q, s, z) in zip(names, gu + dn, outs):
+            words = h.packed_words()
+            done.append((f"{e}.{name}", h))
+            if keep_outputs:
+                res.packed[f"{e}.{name}"] = words
+                res.scales[f"{e}.{name}"] = s
+            if e in keep_codes:
+                res.qweight[f"{e}.{name}"] = q
+                res.scales[f"{e}.{name}"] = s
+        for h in gu + dn:  # as quant.py:330: free per-linear state as soon as the linear is done
+            h.H = None
+            h._hessian_inv = h._loop_factor = None
+            h._Qt = None
+            h.W = h.layer.weight
+
+    chunks = [list(range(e0, min(E, e0 + group))) for e0 in range(0, E, group)]
+    t1 = time.perf_counter()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record(main)
+    if overlap:
+        # The Hessians of a chunk of experts are collected on the current stream; as soon as they are complete the
+        # chunk is quantized on a lane of its own while the next chunk's Hessians are collected.  Legal because the
+        # expert forward reads the original weights whatever has been quantized meanwhile (this driver never writes
+        # quantized weights back), which is all the reference's "collect everything first" order is there for.
+        for ci, chunk in enumerate(chunks):
             for e in chunk:
-                g, u, d = handles[e]
-                if e in keep_codes:
-                    g.symmetrize_hessian()
-                    d.symmetrize_hessian()
-                    if g.H is not None:
-                        res.hessians[f"{e}.gate_proj"] = g.H.clone()
-                    if d.H is not None:
-                        res.hessians[f"{e}.down_proj"] = d.H.clone()
-            # gate and up projections of the chunk (one factor per expert, shared), then the down projections
-            gu = [handles[e][i] for e in chunk for i in (0, 1)]
-            names = [(e, n) for e in chunk for n in ("gate_proj", "up_proj")] + [(e, "down_proj") for e in chunk]
-            dn = [handles[e][2] for e in chunk]
-            if group > 1:
-                outs = GPTQ.quantize_many(gu, bits) + GPTQ.quantize_many(dn, bits)
-            else:
-                outs = [h.quantize(bits) for h in gu + dn]
-            for (e, name), h, (q, s, z) in zip(names, gu + dn, outs):
-                words = h.packed_words()
-                done.append((f"{e}.{name}", h))
-                if keep_outputs:
-                    res.packed[f"{e}.{name}"] = words
-                    res.scales[f"{e}.{name}"] = s
-                if e in keep_codes:
-                    res.qweight[f"{e}.{name}"] = q
-                    res.scales[f"{e}.{name}"] = s
-            for h in gu + dn:  # as quant.py:330: free per-linear state as soon as the linear is done
-                h.H = None
-                h._hessian_inv = h._loop_factor = None
-                h._Qt = None
-                h.W = h.layer.weight
+                collect_hessians(e)
+            ready = torch.cuda.Event()
+            ready.record(main)
+            lane = lanes[ci % len(lanes)]
+            lane.wait_event(ready)
+            with torch.cuda.stream(lane):
+                quantize_chunk(chunk)
+        ev1.record(main)
+    else:
+        # ---- phase 1: Hessians of the whole block, phase 2: quantize + pack, chunks round-robin over the lanes
+        for chunk in chunks:
+            for e in chunk:
+                collect_hessians(e)
+        ev1.record(main)
+        sync()
+        for s_ in lanes:
+            if s_ is not main:
+                s_.wait_stream(main)
+        for ci, chunk in enumerate(chunks):
+            with torch.cuda.stream(lanes[ci % len(lanes)]):
+                quantize_chunk(chunk)
     for s_ in lanes:
         if s_ is not main:
             main.wait_stream(s_)
     sync()
+    t_end = time.perf_counter()
+    # time the Hessian work took on its stream (with overlap: while quantization ran beside it), and the rest of the wall
+    res.seconds["hessians_incl_gather_and_forward"] = ev0.elapsed_time(ev1) / 1e3
+    res.seconds["quantize_and_pack"] = (t_end - t1) - res.seconds["hessians_incl_gather_and_forward"]
+    res.overlapped = bool(overlap)
     issues = {"zero_samples": 0, "nan_hessian": 0, "non_invertible": 0}
     for name, h in done:
         raised = [k for k, v in (("zero_samples", h.issue_zero_samples), ("nan_hessian", h.issue_nan_hessian),
@@ -179,7 +214,6 @@ def quantize_moe_layer(
         if raised:
             res.issues_by_linear[name] = raised
     res.factorizations = GPTQ.factor_calls - factor_calls_before
-    res.seconds["quantize_and_pack"] = time.perf_counter() - t2
     res.seconds["total"] = time.perf_counter() - t0
     res.issues = issues
     return res

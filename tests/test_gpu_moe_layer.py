@@ -97,12 +97,15 @@ def test_reduced_layer_every_linear_against_oracle(dev):
             assert torch.equal(res.packed[f"{e}.{proj}"].cpu(), words), (e, proj)
 
 
-def test_layer_run_equals_one_linear_at_a_time(dev):
+@pytest.mark.parametrize("overlap", [True, False])
+def test_layer_run_equals_one_linear_at_a_time(dev, overlap):
     """The quantize phase of the layer driver (several linears in flight, shared factor for gate/up) against plain
     GPTQ handles given the same Hessians and run one after another on one stream: bit-identical codes and scales."""
     x, ids, experts = _reduced_layer(dev, hidden=1024, inter=512, tokens=4096, seed=77)
     E = len(experts)
-    res = quantize_moe_layer(x.to(dev), ids.to(dev), experts, keep_codes=list(range(E)), streams=4)
+    res = quantize_moe_layer(x.to(dev), ids.to(dev), experts, keep_codes=list(range(E)), streams=4, group=2,
+                             overlap=overlap)
+    assert res.overlapped == overlap
     for e in range(E):
         for proj, W in (("gate_proj", experts[e].gate), ("up_proj", experts[e].up), ("down_proj", experts[e].down)):
             lin = torch.nn.Linear(W.shape[1], W.shape[0], bias=False, dtype=W.dtype, device=dev)
