@@ -222,6 +222,15 @@ def test_block_size_none_means_whole_width(dev):
     assert torch.equal(s.cpu(), ref["scale"]) and m >= 0.999 and m128 >= 0.999
 
 
+@pytest.mark.parametrize("R,C,g,act", [(96, 320, 64, False), (70, 200, 100, True), (256, 1000, 125, False)])
+def test_widths_that_are_not_multiples_of_128(dev, R, C, g, act):
+    """The factorisation works on 128-wide blocks: other widths go through an identity-padded copy of H (diag(H, I)
+    factors to diag(R, I)), the loop through its ragged last block."""
+    case = synth.LinearCase(f"odd_{R}x{C}", synth.weight(R, C, 900 + C), synth.activations_outlier(3 * C, C, 901 + C),
+                            group_size=g, act_order=act)
+    _run_case(case, dev, chunks=2)
+
+
 def test_nan_hessian_falls_back(dev):
     W = synth.weight(64, 256, 2)
     h = GPTQ(_layer(W, dev), 128, True)
