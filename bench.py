@@ -28,7 +28,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--streams", type=int, default=2,
+    ap.add_argument("--streams", type=int, default=3,
                     help="groups of independent linears are queued round-robin on this many HIP streams")
     ap.add_argument("--group", type=int, default=8,
                     help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
@@ -286,20 +286,33 @@ def main():
     group = max(1, args.group)
     lanes = [main_stream] + [torch.cuda.Stream(device=dev) for _ in range(n_lanes - 1)]  # the current stream is lane 0
 
+    def batches(k, n_lanes, group):
+        """k steps as grouped batches of at most `group`, the same number of batches on every lane and sizes as equal
+        as possible (a short run must not end with one lane working through a last batch alone)."""
+        if k <= 0:
+            return []
+        rounds = -(-k // (n_lanes * group))
+        nb = min(k, rounds * n_lanes)
+        return [k // nb + (1 if i < k % nb else 0) for i in range(nb)]
+
     def run(k, lanes, group=group):
         for ln in lanes:
             if ln is not main_stream:
                 ln.wait_stream(main_stream)
         last = None
         t_begin = time.perf_counter()
-        for bi, i in enumerate(range(0, k, group)):
+        for bi, size in enumerate(batches(k, len(lanes), group)):
             with torch.cuda.stream(lanes[bi % len(lanes)]):
-                last = steps(min(group, k - i))
+                last = steps(size)
         host_ms[0] = (time.perf_counter() - t_begin) * 1e3 / max(k, 1)
         torch.cuda.synchronize()
         return last
 
     host_ms = [0.0]
+    # set-up, before the warm-up steps: one batch of the timed region's size on every lane, so that each lane's scratch
+    # buffers and the allocator's pools exist (a first allocation synchronises the device) -- not counted as steps
+    prime = batches(args.steps, len(lanes), group)
+    run(len(lanes) * max(prime), lanes, max(prime)) if prime else None
     run(args.warmup, lanes)
     t0 = time.perf_counter()
     out = run(args.steps, lanes)
@@ -478,6 +491,8 @@ def main():
             "workload": "config 1: expert gate_proj 2048x7168 bf16, 8192 calibration tokens, 4-bit sym g128 B128; "
             "step = Hessian SYRK + factorisation + GPTQ loop + int32 packing",
             "R": R, "C": C, "tokens": n, "streams": n_lanes, "linears_per_grouped_call": group,
+            "batches_of_the_timed_steps": batches(args.steps, n_lanes, group),
+            "setup_linears_before_warmup": len(lanes) * max(prime) if prime else 0,
         },
         "ms_per_step_one_stream": round(ms_single, 3),
         "host_queueing_ms_per_step": round(host_issue_ms, 3),
