@@ -33,8 +33,9 @@ namespace {
 
 constexpr int B = 128;
 constexpr int LOOP_BATCH_MAX = 8;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
-static int LOOP_BATCH = 4;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..8;
-                                    // 1, 2, 3, 4: 0.99, 0.83, 0.77, 0.75 ms per 2048x7168 linear in grouped calls of eight)
+static int LOOP_BATCH = 8;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..8;
+                                    // 1, 2, 3, 4, 6, 8: 0.99, 0.83, 0.77, 0.73, 0.71, 0.70 ms per 2048x7168 linear in
+                                    // grouped calls of eight; a lone call: 2.05 ms at 4, 2.2 at 8)
 
 __device__ __forceinline__ float round_dtype(float x, int rd) {
   // branch-free so that the unrolled column steps stay one basic block
