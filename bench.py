@@ -34,10 +34,11 @@ def parse():
                     help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
-    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer", "gemm", "syrk"],
+    ap.add_argument("--workload", default="config1", choices=["config1", "moe_layer", "gemm", "syrk", "overlap"],
                     help="config1 (default, the benchmark line), moe_layer (config 3: whole MoE layer, one pass) or gemm "
                          "(micro-benchmark of the fp32 GEMM core shared by the factorisation and the loop) or syrk (the "
-                         "Hessian kernel beside the vendor library's GEMM on the same operands)")
+                         "Hessian kernel beside the vendor library's GEMM on the same operands) or overlap (how far grouped calls on "
+                         "different HIP streams run beside each other)")
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--tokens", type=int, default=2_097_152)
     ap.add_argument("--check-experts", type=int, default=2, help="moe_layer: experts compared with the CPU oracle")
@@ -236,6 +237,90 @@ def syrk_main(args):
                       "shapes": out}))
 
 
+def overlap_main(args):
+    """How far library calls queued on different HIP streams run beside each other on the chip: every phase of
+    config 1 as grouped calls of eight, six calls dealt round-robin to 1..4 streams; then a call that is one chain of
+    short launches (a lone factorisation, a lone column loop) beside calls that fill the chip (grouped SYRK, grouped
+    factorisation), alone and together.  One JSON line."""
+    import time
+
+    import torch
+
+    from moe_quant_amd import _lib, ops
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    C, R, n, G, NB = 7168, 2048, 8192, 8, 6
+    X = [torch.randn(n, C, device=dev).to(torch.bfloat16) for _ in range(G)]
+
+    def hessians():
+        Hs = [torch.zeros(C, C, device=dev) for _ in range(G)]
+        ops.hessian_syrk_grouped_(Hs, X, [0.0] * G, [2.0 / n] * G)
+        for H in Hs:
+            H.diagonal().add_(0.01 * H.diagonal().mean())
+        return Hs
+
+    Hb = [hessians() for _ in range(NB)]
+    H1 = [Hb[0][0].clone() for _ in range(8)]
+    W = [(torch.randn(R, C, device=dev) * 0.02).to(torch.bfloat16) for _ in range(G)]
+    Fs, _ = ops.factor_chol_grouped([h.clone() for h in Hb[0]])
+    scales = [ops.quant_grid_sym(w, 128, 4, torch.bfloat16)[1] for w in W]
+    srow = [torch.arange(C, device=dev, dtype=torch.int32) // 128 for _ in range(G)]
+    pairs = [[ops.prepare_wt_pair(w) for w in W] for _ in range(NB)]
+    lone = [ops.prepare_wt_pair(W[0]) for _ in range(10)]
+
+    def syrk(b):
+        ops.hessian_syrk_grouped_(Hb[b % NB], X, [0.0] * G, [2.0 / n] * G)
+
+    def chol(b):
+        ops.factor_chol_grouped(Hb[b % NB])
+
+    def loop(b):
+        ops.gptq_loop_chol_grouped_([p[0] for p in pairs[b % NB]], [p[1] for p in pairs[b % NB]], Fs, scales, srow, 8.0, 15.0,
+                                    torch.bfloat16, 128)
+
+    def chol1(i):
+        ops.factor_chol(H1[i % 8])
+
+    def loop1(i):
+        ops.gptq_loop_chol_grouped_([lone[i % 10][0]], [lone[i % 10][1]], [Fs[0]], [scales[0]], [srow[0]], 8.0, 15.0,
+                                    torch.bfloat16, 128)
+
+    streams = [torch.cuda.Stream(device=dev) for _ in range(4)]
+
+    def wall(plan):  # plan: (function, argument, stream index); best of three after one untimed pass
+        best = None
+        for it in range(4):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for fn, a, si in plan:
+                with torch.cuda.stream(streams[si]):
+                    fn(a)
+            torch.cuda.synchronize()
+            t = (time.perf_counter() - t0) * 1e3
+            if it and (best is None or t < best):
+                best = t
+        return round(best, 2)
+
+    out = {"ms_per_linear_by_streams": {}, "chain_beside_full_chip_ms": {}}
+    kinds = {"syrk": [syrk], "factor": [chol], "loop": [loop], "factor+loop": [chol, loop], "syrk+factor+loop": [syrk, chol, loop]}
+    for name, fns in kinds.items():
+        calls = [(f, b) for b in range(NB) for f in fns]
+        out["ms_per_linear_by_streams"][name] = {
+            str(S): round(wall([(f, b, i % S) for i, (f, b) in enumerate(calls)]) / (NB * G), 3) for S in (1, 2, 3, 4)}
+    for (na, fa, ca), (nb_, fb, cb) in ((("syrk x8", syrk, 6), ("lone factor", chol1, 7)),
+                                        (("syrk x8", syrk, 6), ("lone loop", loop1, 10)),
+                                        (("factor x8", chol, 3), ("lone factor", chol1, 7)),
+                                        (("factor x8", chol, 3), ("lone loop", loop1, 10))):
+        a = wall([(fa, i, 0) for i in range(ca)])
+        b = wall([(fb, i, 1) for i in range(cb)])
+        ab = wall([(fa, i, 0) for i in range(ca)] + [(fb, i, 1) for i in range(cb)])
+        out["chain_beside_full_chip_ms"][f"{ca} calls of {na} | {cb} calls of {nb_}"] = {"first_alone": a, "second_alone": b, "together": ab}
+    print(json.dumps({"metric": "wall time of config-1 library calls queued on several HIP streams", "unit": "ms", "n_gpus": 1,
+                      "data": "synthetic", "linears_per_grouped_call": G, **out}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -247,6 +332,8 @@ def main():
         return gemm_main(args)
     if args.workload == "syrk":
         return syrk_main(args)
+    if args.workload == "overlap":
+        return overlap_main(args)
     import torch
 
     from moe_quant_amd import _lib, ops, synth
@@ -365,6 +452,10 @@ def main():
     t_pack = timed(lambda: ops.pack_from_qt(Qt), reps=10)
     codes = ops.untranspose_codes(Qt)
     t_pack_rc = timed(lambda: ops.pack_int4(codes), reps=10)
+    # one launch of 22 MB is launch latency; the kernel's own rate shows on sixteen linears' codes stacked into one launch
+    codes16 = codes.repeat(16, 1)
+    t_pack16 = timed(lambda: ops.pack_int4(codes16), reps=10)
+    del codes16
 
     # the three big phases once more as the step runs them: one grouped library call over `group` linears on one
     # stream; device time of the call / group
@@ -415,6 +506,8 @@ def main():
         "gptq_loop_tflops": round(flop_loop / t_loop / 1e9, 2),
         "pack_int4_gbps": round(bytes_pack / t_pack_rc / 1e6, 1),
         "pack_int4_frac_hbm_peak": round(bytes_pack / t_pack_rc / 1e6 / PEAK_HBM, 4),
+        "pack_int4_gbps_16_linears_one_launch": round(16 * bytes_pack / t_pack16 / 1e6, 1),
+        "pack_int4_frac_hbm_peak_16_linears_one_launch": round(16 * bytes_pack / t_pack16 / 1e6 / PEAK_HBM, 4),
     }
     # Dominant call of the step: the factorisation, as the step runs it -- one grouped call over `group` matrices
     # (one "launch" = one call = a fixed sequence of kernels, each carrying the work of all matrices).
