@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--experts", type=int, default=256)
     ap.add_argument("--tokens", type=int, default=2_097_152)
     ap.add_argument("--check-experts", type=int, default=2, help="moe_layer: experts compared with the CPU oracle")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="moe_layer: the reference's order, every Hessian of the layer first, then quantization (kernel "
+                         "durations in a profiler trace are then not stretched by kernels of the other streams)")
     ap.add_argument("--no-moe-layer", action="store_true",
                     help="config1: skip the one pass over the whole MoE layer (config 3) reported next to the headline")
     return ap.parse_args()
@@ -85,7 +88,7 @@ def moe_layer_run(args, with_cpu_oracle=True):
     quantize_moe_layer(x[:4096], ids[:4096] % 2, experts[:2])
     counts = torch.bincount(ids.flatten(), minlength=args.experts)
     check = torch.argsort(counts, descending=True)[: args.check_experts].tolist() if args.check_experts else []
-    res = quantize_moe_layer(x, ids, experts, keep_codes=check)
+    res = quantize_moe_layer(x, ids, experts, keep_codes=check, overlap=not getattr(args, "no_overlap", False))
     C, I = x.shape[1], experts[0].gate.shape[0]
     n_e = torch.tensor(res.tokens_per_expert, dtype=torch.float64)
     flop_syrk = float((n_e * (C * (C + 1) + I * (I + 1))).sum())
