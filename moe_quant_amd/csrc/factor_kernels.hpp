@@ -27,7 +27,9 @@
 
 #include "gemm_f32_tile.hpp"
 
+// (internal linkage: each translation unit that includes this header gets its own kernels and tuning knobs)
 namespace mqfactor {
+namespace {
 
 constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
@@ -817,4 +819,5 @@ struct FactorPlan {
   }
 };
 
+}  // namespace
 }  // namespace mqfactor

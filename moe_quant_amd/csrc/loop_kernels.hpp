@@ -31,7 +31,9 @@
 
 #include "gemm_f32_tile.hpp"
 
+// (internal linkage: each translation unit that includes this header gets its own kernels and tuning knobs)
 namespace mqloop {
+namespace {
 
 constexpr int B = 128;
 constexpr int LOOP_BATCH_MAX = 8;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
@@ -635,4 +637,5 @@ inline int make_plan(LoopPlan& p, int G, float* const* Wt, long ldw, int C, int 
   return MQ_OK;
 }
 
+}  // namespace
 }  // namespace mqloop
