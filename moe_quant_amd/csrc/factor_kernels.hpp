@@ -35,8 +35,24 @@ constexpr int NB = 128;
 constexpr int SB = 32;     // sub-block edge inside the diagonal-block kernel
 constexpr int LDM = 132;   // LDS row pitch: rows 16-byte aligned, consecutive rows 4 banks apart (8 rows span the 32 banks)
 constexpr int SOFF = 4;    // column shift of the S triangle inside a row (keeps both triangles 16-byte aligned)
-inline int TRAIL_PANELS = 8;  // panels per trailing update of the whole matrix (env MQ_PANELS)
-inline int INV_KC = 4;  // the first inverse product is cut into K chunks of 4 blocks (512), one workgroup each
+// Tuning knobs, read from the environment once (function-local statics: safe whichever host thread asks first).
+inline int env_knob(const char* name, int dflt) {
+  if (const char* e = getenv(name)) {
+    const int v = atoi(e);
+    if (v > 0) return v;
+  }
+  return dflt;
+}
+// panels per trailing update of the whole matrix (env MQ_PANELS)
+inline int trail_panels() {
+  static const int v = env_knob("MQ_PANELS", 8);
+  return v;
+}
+// the first inverse product is cut into K chunks of this many blocks (4 = 512 deep), one workgroup each (env MQ_INV_KC)
+inline int inv_kc() {
+  static const int v = env_knob("MQ_INV_KC", 4);
+  return v;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Diagonal block: S (128x128, upper valid) -> R^-1 where S = R R^T, R upper.
@@ -691,12 +707,10 @@ struct FactorPlan {
     return MQ_OK;
   }
 
-  // kernel attributes and tuning knobs: set once, whichever host thread comes first
+  // kernel attributes: set once, whichever host thread comes first
   static void init_kernels() {
     static std::once_flag once;
     std::call_once(once, [] {
-      if (const char* e = getenv("MQ_INV_KC")) INV_KC = atoi(e) > 0 ? atoi(e) : INV_KC;
-      if (const char* e = getenv("MQ_PANELS")) TRAIL_PANELS = atoi(e) > 0 ? atoi(e) : TRAIL_PANELS;
       (void)hipFuncSetAttribute((const void*)revchol_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)DIAG_SMEM);
       (void)hipFuncSetAttribute((const void*)trail_diag_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -708,7 +722,7 @@ struct FactorPlan {
     });
   }
 
-  int kc_of(int) const { return INV_KC; }  // one depth for all block rows: 2, 3 for the short rows measured no faster
+  int kc_of(int) const { return inv_kc(); }  // one depth for all block rows: 2, 3 for the short rows measured no faster
   // the two products of block row b of the inverse (w = columns to the right of b)
   GemmF32 inv_first(int b, int& tiles) const {  // T^T (w x 128) = U22^T (w x w) * R12^T (w x 128), in K chunks
     const long p = (long)b * NB;
@@ -753,11 +767,11 @@ struct FactorPlan {
   // The trailing launch of step s: fills T, returns its number of workgroups.
   // The trailing update A[0:i1,0:i1] -= P P^T with one 128-wide panel is bound by reading and writing the
   // trailing matrix, so after the first step (which also carries the matrix from S to A) the panels go in
-  // TRAIL_PANELS at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0
+  // trail_panels() at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0
   // owns its diagonal tile.  Steps in between (column_only): the j panels block column b-1 still lacks --
   // this one and the j-1 before it, neighbours in memory, A[:, i1 : i1+128j], one product with K = 128j --
   // into that block column alone, and already into the diagonal tile after the next one, (b-2, b-2).  Every
-  // TRAIL_PANELS-th step: the last TRAIL_PANELS panels into every tile but (b-1, b-1), which had all but
+  // trail_panels()-th step: the last trail_panels() panels into every tile but (b-1, b-1), which had all but
   // this panel one step early and takes this one from workgroup 0 as always.
   // (2, 3, 4, 6 panels: 306, 311, 314, 315 linears/s at four streams against 286 with one; a single
   // factorisation takes 3.21 -> 3.28 ms with four, the steps in between leave the chip idle.)
@@ -765,8 +779,9 @@ struct FactorPlan {
     const int b = B - 1 - s, i1 = b * NB, G = grp.n;
     float* P = A + i1;
     const bool first = (b == B - 1) && !in_place;
-    const int j = s >= 1 ? (s - 1) % TRAIL_PANELS + 1 : 1;  // panels owed to block column b-1 (step 0: the plain update)
-    const int column_only = s >= 1 && j < TRAIL_PANELS;
+    const int TP = trail_panels();
+    const int j = s >= 1 ? (s - 1) % TP + 1 : 1;  // panels owed to block column b-1 (step 0: the plain update)
+    const int column_only = s >= 1 && j < TP;
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, j * NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
     if (first) {
       trail.Csrc = S0;

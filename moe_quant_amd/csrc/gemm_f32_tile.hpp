@@ -332,15 +332,13 @@ __device__ __forceinline__ void split3(const floatx4 v, uint2v& hi, uint2v& mid,
 template <bool KC>
 struct Loader {
   floatx4 r[2];
-  // element (x, k) at p[x*sx + k*sk]; KC: sk == 1, else sx == 1
-  __device__ __forceinline__ const float* addr(const float* p, long sx, long sk, int x0, int k0, int it, int tid) const {
+  // element (x, k) at p[x*sx + k*sk]; KC: sk == 1, else sx == 1.  X: the operand's extent along x; a tile that
+  // sticks out past it fetches the last valid row (or quad of rows) again in place of what does not exist --
+  // an address clamp, no branch -- and the caller never stores the results computed from those.
+  __device__ __forceinline__ const float* addr(const float* p, long sx, long sk, int x0, int X, int k0, int it, int tid) const {
     const int idx = tid + it * 256;
-    if (KC) return p + (long)(x0 + (idx >> 2)) * sx + k0 + ((idx & 3) << 2);
-    return p + (long)(k0 + (idx >> 5)) * sk + x0 + ((idx & 31) << 2);
-  }
-  __device__ __forceinline__ void load(const float* __restrict__ p, long sx, long sk, int x0, int k0, int tid) {
-#pragma unroll
-    for (int it = 0; it < 2; ++it) r[it] = *reinterpret_cast<const floatx4*>(addr(p, sx, sk, x0, k0, it, tid));
+    if (KC) return p + (long)min(x0 + (idx >> 2), X - 1) * sx + k0 + ((idx & 3) << 2);
+    return p + (long)(k0 + (idx >> 5)) * sk + min(x0 + ((idx & 31) << 2), X - 4);
   }
   __device__ __forceinline__ void store(unsigned char* op, int tid) const {
 #pragma unroll
@@ -420,8 +418,8 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
   const float* qb[2];
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
-    qa[it] = la[0].addr(A, g.sam, g.sak, m0, kb, it, tid);
-    qb[it] = lb[0].addr(B, g.sbn, g.sbk, n0, kb, it, tid);
+    qa[it] = la[0].addr(A, g.sam, g.sak, m0, g.M, kb, it, tid);
+    qb[it] = lb[0].addr(B, g.sbn, g.sbk, n0, g.N, kb, it, tid);
   }
   const long inca = (long)SBK * g.sak, incb = (long)SBK * g.sbk;
   int fetched = 0;  // steps fetched so far
@@ -449,7 +447,8 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
 #pragma unroll
     for (int it = 0; it < 16; ++it) {
       const int idx = tid + it * 256;
-      cold4[it] = *reinterpret_cast<const floatx4*>(Cold + (long)(m0 + (idx >> 5)) * ldcold + n0 + ((idx & 31) << 2));
+      cold4[it] = *reinterpret_cast<const floatx4*>(Cold + (long)min(m0 + (idx >> 5), g.M - 1) * ldcold +
+                                                    min(n0 + ((idx & 31) << 2), g.N - 4));
     }
   }
   if (nk > 0) {
@@ -508,7 +507,7 @@ __device__ __forceinline__ void tile_core_split(const GemmF32& g, int m0, int n0
       if (beta != 0.f) x = fmaf(beta, cold4[it][e], x);
       o[e] = x;
     }
-    *reinterpret_cast<floatx4*>(C + (long)(m0 + r) * g.ldc + n0 + c) = o;
+    if (m0 + r < g.M && n0 + c < g.N) *reinterpret_cast<floatx4*>(C + (long)(m0 + r) * g.ldc + n0 + c) = o;
   }
 }
 
@@ -651,7 +650,11 @@ __device__ __forceinline__ void tile_body(const GemmF32& g, int tm, int tn, int 
   const bool c_vec = LDS_OUT || ((((uintptr_t)C) & 15) == 0 && (g.ldc & 3) == 0 &&  // C moves 16 bytes at a time
                                  (!g.Csrc || ((((uintptr_t)g.Csrc) & 15) == 0 && (g.ldcs & 3) == 0)));
   const bool inside = vecA && vecB && c_vec && m0 + BM <= g.M && n0 + BN <= g.N;
-  if (!LDS_OUT && !g.fp32_mfma && !g.bsum && inside && ((ke - kb) % split::SBK == 0)) {
+  // a tile that sticks out of the matrix still takes the fast path when whole quads of rows and columns exist (its
+  // loads clamp their addresses, its stores are masked): K-contiguous operands need nothing, the others and C move
+  // four elements of M or N at a time
+  const bool quads = vecA && vecB && c_vec && g.M >= 4 && g.N >= 4 && (g.N & 3) == 0 && (A_KC || (g.M & 3) == 0);
+  if (!LDS_OUT && !g.fp32_mfma && !g.bsum && (inside || quads) && ((ke - kb) % split::SBK == 0)) {
     tile_core_split<A_KC, B_KC>(g, m0, n0, kb, ke, A, B, C, smem);
     return;
   }

@@ -37,9 +37,19 @@ namespace {
 
 constexpr int B = 128;
 constexpr int LOOP_BATCH_MAX = 8;   // the caller's E holds a ring of 2 * LOOP_BATCH_MAX error blocks
-inline int LOOP_BATCH = 8;          // blocks of errors per trailing update of everything beyond (env MQ_LOOP_BATCH, 1..8;
-                                    // 1, 2, 3, 4, 6, 8: 0.99, 0.83, 0.77, 0.73, 0.71, 0.70 ms per 2048x7168 linear in
-                                    // grouped calls of eight; a lone call: 2.05 ms at 4, 2.2 at 8)
+// blocks of errors per trailing update of everything beyond: 8, or env MQ_LOOP_BATCH (1..8), read once (a function-local
+// static: safe whichever host thread asks first).  1, 2, 3, 4, 6, 8: 0.99, 0.83, 0.77, 0.73, 0.71, 0.70 ms per 2048x7168
+// linear in grouped calls of eight; a lone call: 2.05 ms at 4, 2.2 at 8.
+inline int loop_batch() {
+  static const int v = [] {
+    if (const char* e = getenv("MQ_LOOP_BATCH")) {
+      const int x = atoi(e);
+      if (x >= 1 && x <= LOOP_BATCH_MAX) return x;
+    }
+    return 8;
+  }();
+  return v;
+}
 
 __device__ __forceinline__ float round_dtype(float x, int rd) {
   // branch-free so that the unrolled column steps stay one basic block
@@ -531,9 +541,9 @@ struct LoopPlan {
     L.i1 = i1;
     L.nb = nb;
     L.col_wgs = grid;
-    // Error blocks live in a ring of 2 * LOOP_BATCH: this block's, the previous one (the column workgroups fold it
+    // Error blocks live in a ring of 2 * loop_batch(): this block's, the previous one (the column workgroups fold it
     // into their own columns) and the batches a trailing update may still be reading.
-    const int RING = 2 * LOOP_BATCH;  // a multiple of the batch: an aligned batch never wraps
+    const int RING = 2 * loop_batch();  // a multiple of the batch: an aligned batch never wraps
     LoopOffsets& off = L.off;
     off.e_cur = (long)(blk % RING) * B * a.R;
     off.e_prev = blk ? (long)((blk - 1) % RING) * B * a.R : -1;
@@ -555,7 +565,7 @@ struct LoopPlan {
       long j0 = i1 - nbprev;
       off.g_b = off.e_prev;
       if (block == B) {
-        const int D = LOOP_BATCH, r = blk % D;
+        const int D = loop_batch(), r = blk % D;
         const int first = r ? blk - r : blk - D;  // first block of the errors applied now
         if (r) g.M = (a.C - i2 < block) ? a.C - i2 : block;
         j0 = (long)first * B;
@@ -576,7 +586,7 @@ struct LoopPlan {
   }
 };
 
-// kernel attributes and the tuning knob: once per template instance, whichever host thread comes first
+// kernel attributes: once per template instance, whichever host thread comes first
 template <bool ROWMAP, bool QZERO, bool ZMODE>
 inline void init_loop_kernels() {
   static std::once_flag once;
@@ -585,10 +595,6 @@ inline void init_loop_kernels() {
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
     (void)hipFuncSetAttribute((const void*)gptq_block_kernel<false, ROWMAP, QZERO, ZMODE>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLOCK_SMEM);
-    if (const char* e = getenv("MQ_LOOP_BATCH")) {
-      const int v = atoi(e);
-      if (v >= 1 && v <= LOOP_BATCH_MAX) LOOP_BATCH = v;
-    }
   });
 }
 

@@ -30,7 +30,9 @@ class QuantizationOrder(Enum):
 class GPTQ:
     """Mirror of src/gptq.py:22-243 (constructor arguments, attributes and methods keep their names)."""
 
-    factor_calls = 0  # factorisations computed so far by all handles (a tied handle that reuses its owner's adds none)
+    # factorisations computed so far by all handles (a tied handle that reuses its owner's adds none); a plain class
+    # counter for tests and logs, not synchronised between host threads
+    factor_calls = 0
 
     def __init__(
         self,
@@ -195,14 +197,21 @@ class GPTQ:
             self.H = None
             self._hessian_inv = self._loop_factor = None
             self._H_upper_only = self._H_clean = False
+            self._perm = None
         elif self.tied_gptq_handle:
             self.tied_gptq_handle.num_tied_handles -= 1
             if self.tied_gptq_handle.num_tied_handles == 0:
                 self.tied_gptq_handle.H = None
                 self.tied_gptq_handle._hessian_inv = self.tied_gptq_handle._loop_factor = None
                 self.tied_gptq_handle._H_upper_only = self.tied_gptq_handle._H_clean = False
+                self.tied_gptq_handle._perm = None
+        # (while tied handles still need this handle's H -- permuted in place under act-order -- the column order that
+        # goes with it is kept as well, like H and the factor: whether the owner is reset before its tied handles are
+        # quantized, as the reference's driver does (quant.py:297-330), or after, they pair permuted weights with the
+        # permuted H.  The reference re-sorts the already sorted diagonal there and pairs un-permuted weights with it.)
         self.num_samples = 0
-        self._perm = None
+        if self.tied_gptq_handle is not None:
+            self._perm = None
         self._pruned = None
         if self.tied_gptq_handle is not None:
             self._hessian_inv = self._loop_factor = None
@@ -345,7 +354,8 @@ class GPTQ:
         """`[h.quantize(bits) for h in handles]` for linears of one shape and one configuration (the experts of a
         block, which the reference quantizes one after another, quant.py:291-386), with the two long phases --
         factorisation and column loop -- run as one grouped library call each: a lone factorisation or loop is a
-        chain of dependent launches that cannot fill the GPU.  Same results, bit for bit, as one call per handle.
+        chain of dependent launches that cannot fill the GPU.  Same results, bit for bit, as one call per handle,
+        with or without a `reset()` of the owner between the calls.
         A tied handle must come after its owner (in this list or in an earlier call)."""
         handles = list(handles)
         if not handles:

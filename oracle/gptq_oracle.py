@@ -234,9 +234,12 @@ def gptq_loop(
     gptq_block_size: int = 128,
     half_up: bool = True,
     fused: bool = True,
+    pre: Optional[Tensor] = None,
 ) -> Tensor:
     """weight (C,R) fp32 is modified in place to the dequantized values; returns codes (C,R) fp32.
-    Mirrors gptq_loop_graph(direct=True), src/gptq_loop.py:141-148."""
+    Mirrors gptq_loop_graph(direct=True), src/gptq_loop.py:141-148.
+    pre (optional, (C,R) fp32): receives every column as it stands when its turn to be quantized comes (a
+    by-product for tests that ask how close a rounding decision was; the arithmetic is untouched)."""
     C, R = weight.shape
     if gptq_block_size <= 0:  # src/gptq_loop.py:212-213
         gptq_block_size = C
@@ -246,6 +249,8 @@ def gptq_loop(
         i2 = min(i1 + gptq_block_size, C)
         for j in range(i1, i2):
             x = weight[j]
+            if pre is not None:
+                pre[j] = x
             q = quantize(x, scale[j], qzero[j], maxq, half_up)  # tl_quantize, src/gptq_loop.py:34
             y = dequantize(q, scale[j], qzero[j], dtype)  # tl_dequantize, :35
             e = y - x  # :36
@@ -280,31 +285,40 @@ def quantize_linear(
     half_up: bool = True,
     inverse_dtype=torch.float32,
     mse: bool = False,
+    keep_pre: bool = False,
+    perm: Optional[Tensor] = None,
 ):
-    """Returns dict(qweight u8 (R,C), scale (R,G), zero (R,G), U, perm, H (damped, permuted), ok)."""
+    """Returns dict(qweight u8 (R,C), scale (R,G), zero (R,G), U, perm, H (damped, permuted), ok).
+    keep_pre: also `tie_distance` (R,C) fp32 in the original column order: how far x/s + zero + 0.5 was from the
+    nearest integer when the column was quantized (0 = an exact tie of the rounding decision).
+    perm: with act_order, the column order to use in place of this function's own argsort (src/gptq.py:181 sorts with
+    an unstable sort: where diag(H) holds equal values their order is open, and a test that compares with a device run
+    passes the order the device chose)."""
     dtype = dtype or W.dtype
     R, C = W.shape
     H, W32, zero_samples, nan_h = quantization_pre_step(H, W)
     g = group_size or C
     scale_g, zero_g, maxq = quantization_grid(W32, g, bits, dtype, mse=mse)  # src/gptq.py:171-178
     scale, zero = replicate_grid(scale_g, zero_g, g)
-    perm, perm_inv = act_order_perm(H, act_order)
+    if perm is not None and act_order:
+        perm_inv = torch.argsort(perm)
+    else:
+        perm, perm_inv = act_order_perm(H, act_order)
     H = H[perm][:, perm]  # src/gptq.py:187
     U, ok = hessian_inverse(H, W32, rel_damp, inverse_dtype)  # :189
     U = U.float()
     Wt = W32.t()[perm].contiguous()  # :192
-    q = gptq_loop(
-        Wt,
-        U,
-        scale.t()[perm].contiguous(),
-        zero.t()[perm].contiguous(),
-        maxq,
-        dtype,
-        block_size or C,
-        half_up,
-    )
+    st, zt = scale.t()[perm].contiguous(), zero.t()[perm].contiguous()
+    pre = torch.empty_like(Wt) if keep_pre else None
+    q = gptq_loop(Wt, U, st, zt, maxq, dtype, block_size or C, half_up, pre=pre)
     qweight = q[perm_inv].t().contiguous().to(torch.uint8)  # :199
+    extra = {}
+    if keep_pre:
+        v = pre / st + zt + 0.5
+        extra["tie_distance"] = (v - torch.round(v)).abs()[perm_inv].t().contiguous()
+        extra["order_position"] = perm_inv  # position of original column c in the loop's walking order
     return dict(
+        **extra,
         qweight=qweight,
         scale=scale[:, ::g].to(dtype),  # :201
         zero=zero[:, ::g].to(dtype),  # :202

@@ -27,7 +27,20 @@ def _layer(W, dev):
     return layer
 
 
-def _run_case(case, dev, chunks=3, code_gate=0.999):
+def first_differences_tie_distance(q, ref):
+    """For every row whose codes differ from the oracle's: how close the oracle's own rounding decision was
+    (|x/s + zero + 0.5 - nearest integer|) at the FIRST differing column in the loop's walking order.  Sums taken in
+    another order move x by a few ulps and can only flip decisions that were that close; a defect (wrong index, wrong
+    multiplier, dropped term) flips decisions that were not.  Later differences in a row are consequences of the first."""
+    diff = q != ref["qweight"]
+    C = diff.shape[1]
+    pos = ref["order_position"][None, :].expand_as(diff)
+    first = torch.where(diff, pos, torch.full_like(pos, C)).argmin(dim=1)
+    rows = diff.any(dim=1)
+    return ref["tie_distance"][rows, first[rows]]
+
+
+def _run_case(case, dev, chunks=3, code_gate=0.999, same_h_gate=0.9995, tie_tol=1e-3):
     _say(f"case {case.name} W{tuple(case.W.shape)} X{tuple(case.X.shape)} g={case.group_size} act={case.act_order}")
     h = GPTQ(_layer(case.W, dev), group_size=case.group_size, sym=True, rel_damp=case.rel_damp,
              block_size=case.block_size, quantization_order="activation" if case.act_order else "default")
@@ -39,10 +52,31 @@ def _run_case(case, dev, chunks=3, code_gate=0.999):
     H64 = O.hessian_fp64([case.X])
     h.symmetrize_hessian()
     herr = ((h.H.cpu().double() - H64).norm() / H64.norm()).item()
+    H_gpu = h.H.cpu()
     q, s, z = h.quantize(4)
     ref = O.quantize_linear(case.W, Href.clone(), group_size=case.group_size, rel_damp=case.rel_damp,
                             block_size=case.block_size, act_order=case.act_order)
     match = (q.cpu() == ref["qweight"]).float().mean().item()
+    # The same comparison with the Hessian taken out of the equation: the oracle run on the very matrix the GPU
+    # accumulated.  What is left is factorisation + loop, gated tighter than the end-to-end figure; and every row's
+    # first difference must sit on a rounding decision the oracle itself found close.
+    # (act-order: diag(H) holds exactly equal fp32 values once there are a thousand channels, and torch.argsort leaves
+    # their order open -- the CPU's and the device's sort may differ there.  The oracle gets the order the device chose,
+    # after checking that it is a valid descending order of that diagonal.)
+    perm_dev = None
+    if case.act_order:
+        perm_dev = h._perm.cpu()
+        d = H_gpu.diag()[perm_dev]
+        assert bool((d[:-1] >= d[1:]).all()) and torch.equal(torch.sort(perm_dev).values, torch.arange(d.numel()))
+        _say(f"  act-order: {int((d[:-1] == d[1:]).sum())} pairs of equal neighbours in the sorted diagonal")
+    same = O.quantize_linear(case.W, H_gpu, group_size=case.group_size, rel_damp=case.rel_damp, block_size=case.block_size,
+                             act_order=case.act_order, keep_pre=True, perm=perm_dev)
+    match_same = (q.cpu() == same["qweight"]).float().mean().item()
+    td = first_differences_tie_distance(q.cpu(), same)
+    _say(f"  same Hessian: code match {match_same:.6f}; rows that differ {td.numel()}, largest tie distance at a first "
+         f"difference {td.max().item() if td.numel() else 0.0:.2e}")
+    assert match_same >= same_h_gate
+    assert td.numel() == 0 or td.max().item() < tie_tol
     Wd = case.W.double()
     e_hip = O.relative_mse(O.dequantize_linear_weight(q.cpu(), s.cpu(), z.cpu()).double(), Wd, H64).item()
     e_ref = O.relative_mse(O.dequantize_linear_weight(ref["qweight"], ref["scale"], ref["zero"]).double(), Wd, H64).item()
@@ -94,7 +128,7 @@ def _full_size_properties(dev, R, C, n, g, act_order, seed):
     (3) scales equal the oracle's closed form; codes in range; packed words unpack to the codes; (4) rows are
     independent: quantizing the first 256 rows alone gives the same codes bit for bit; (5) the GPTQ codes beat
     round-to-nearest on the layer-output error tr(dH d^T)."""
-    from moe_quant_amd import linalg_utils
+    from moe_quant_amd import linalg_utils, ops
 
     _say(f"full-size properties R={R} C={C} n={n} g={g} act_order={act_order}")
     gen = torch.Generator(device=dev).manual_seed(seed)
@@ -124,7 +158,19 @@ def _full_size_properties(dev, R, C, n, g, act_order, seed):
     d = T.diagonal().clone()
     T.diagonal().zero_()
     assert (T.norm() / d.norm()).item() < 1e-3
-    del T, U
+    # ... and the multipliers F = -R[j,k]/R[k,k] the quantize path actually hands to the loop (H = R R^T): with
+    # M = I - triu(F, 1) = R diag(R)^-1 and U = diag(R) R^-1 (rows of R^-1 divided by their diagonal), U M = I.
+    F, finfo = ops.factor_chol(h.H)
+    assert int(finfo.item()) == 0
+    M = -torch.triu(F, 1)
+    M.diagonal().fill_(1.0)
+    del F
+    P = U @ M
+    P.diagonal().sub_(1.0)
+    dev_I = (P.norm() / C**0.5).item()
+    _say(f"  |U (I - triu(F,1)) - I|_F / sqrt(C) = {dev_I:.2e}")
+    assert dev_I < 1e-3
+    del T, U, M, P
     # (3)
     sc_ref = O.find_quantization_meta(W.cpu().float().reshape(R, C // g, g), 4, torch.bfloat16)[0]
     assert torch.equal(s.cpu().float(), sc_ref.reshape(R, C // g).float())
@@ -151,8 +197,20 @@ def test_config4_o_proj_full_size_properties(dev):
     _full_size_properties(dev, 7168, 16384, 16384, 128, False, 4400)
 
 
+def test_config4_q_b_proj_full_size_properties(dev):
+    _full_size_properties(dev, 24576, 1536, 16384, 128, False, 4410)
+
+
+def test_config4_kv_b_proj_full_size_properties(dev):
+    _full_size_properties(dev, 32768, 512, 16384, 128, False, 4430)
+
+
 def test_config5_gate_up_full_size_properties(dev):
     _full_size_properties(dev, 18432, 7168, 65536, 64, True, 5500)
+
+
+def test_config5_gate_up_g32_full_size_properties(dev):
+    _full_size_properties(dev, 18432, 7168, 65536, 32, True, 5520)
 
 
 def test_config5_down_full_size_properties(dev):
@@ -285,6 +343,33 @@ def test_tied_handles_share_hessian_and_factor(dev):
     assert (qg.cpu() == O.quantize_linear(Wg, Href.clone())["qweight"]).float().mean().item() >= 0.999
     assert (qu.cpu() == O.quantize_linear(Wu, Href.clone())["qweight"]).float().mean().item() >= 0.999
     up.reset()
+
+
+def test_tied_act_order_in_the_reference_drivers_call_order(dev):
+    """quant.py:297-330 quantizes and resets gate_proj before it quantizes the tied up_proj.  Under act-order the
+    owner's H is permuted in place; the tied handle must get the owner's column order in that call order too (and the
+    same bits as when both are quantized in one grouped call, where no reset comes in between)."""
+    Wg, Wu = synth.weight(128, 384, 17), synth.weight(128, 384, 18)
+    X = synth.activations_outlier(900, 384, 19)
+
+    def pair():
+        g = GPTQ(_layer(Wg, dev), 128, True, 0.01, 128, quantization_order="activation")
+        u = GPTQ(_layer(Wu, dev), 128, True, 0.01, 128, quantization_order="activation", tied_gptq_handle=g)
+        g.update(X.to(dev))
+        return g, u
+
+    g, u = pair()
+    qg, _, _ = g.quantize(4)
+    g.reset()
+    assert g.H is not None and g._perm is not None  # both still owed to the tied handle
+    qu, su, _ = u.quantize(4)
+    u.reset()  # (as in the reference, src/gptq.py:111-118, a tied handle's reset never releases the owner's H)
+    g2, u2 = pair()
+    (qg2, _, _), (qu2, su2, _) = GPTQ.quantize_many([g2, u2], 4)
+    assert torch.equal(qg, qg2) and torch.equal(qu, qu2) and torch.equal(su, su2)
+    Href, _ = O.hessian_update(None, 0, X)
+    ref = O.quantize_linear(Wu, Href.clone(), act_order=True)  # the pairing a lone act-order handle would get
+    assert (qu.cpu() == ref["qweight"]).float().mean().item() >= 0.999
 
 
 def test_mse_scale_option_end_to_end(dev):

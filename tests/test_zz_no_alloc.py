@@ -42,6 +42,21 @@ def test_noalloc_damp_equals_workspace_damp_twice_second_smaller(dev):
     _both(dev, 200, 1000, 3, torch.float32)  # unaligned width, fp32 weights: the scalar scan path
 
 
+def test_noalloc_damp_allocates_nothing(dev):
+    """What the entry point is for: after the first call on a device (which looks up the scratch array's address),
+    a call neither takes memory from torch's allocator nor from the device behind its back."""
+    H, W = _problem(dev, 128, 768, 4)
+    pruned, flags = ops.hessian_prestep_(H, False)
+    ops.hessian_damp_noalloc_(H, W, pruned, 0.01, flags)  # first call: the one-time symbol lookup
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0])
+    for _ in range(3):
+        ops.hessian_damp_noalloc_(H, W, pruned, 0.01, flags)
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0])
+    assert before == after, (before, after)
+
+
 def test_noalloc_damp_refuses_what_does_not_fit(dev):
     lib = _lib.load()
     flags = torch.zeros(4, dtype=torch.int32, device=dev)
