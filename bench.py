@@ -46,6 +46,10 @@ def parse():
     ap.add_argument("--no-overlap", action="store_true",
                     help="moe_layer: the reference's order, every Hessian of the layer first, then quantization (kernel "
                          "durations in a profiler trace are then not stretched by kernels of the other streams)")
+    ap.add_argument("--only", default=None, help="config4 / config5: run just the linear of this name (e.g. o_proj, down_g128)")
+    ap.add_argument("--plain", action="store_true",
+                    help="config2 / config4 / config5: whole steps only (one warm-up + --reps), no per-phase timing passes")
+    ap.add_argument("--reps", type=int, default=0, help="config2 / config4 / config5: timed repetitions per linear (0 = default)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="config1: skip the lone linears of configs 2, 4 and 5 reported next to the headline")
     ap.add_argument("--no-moe-layer", action="store_true",
@@ -109,6 +113,9 @@ def device_inputs(dev, R, C, n, seed, x_kind="outlier"):
     return W, X
 
 
+PLAIN = [False]  # --plain: the lone-linear workloads run whole steps only (one warm-up + reps), for profiler runs
+
+
 def linear_leg(dev, name, R, C, n, g, act_order, x_kind="outlier", seed=0, reps=3, profile_key=None):
     """One linear quantized alone on the GPU -- the regime of a block's attention, dense-MLP and shared-expert linears,
     which the reference quantizes one by one (quant.py:291-330) and which have no sibling of the same shape to share
@@ -141,6 +148,9 @@ def linear_leg(dev, name, R, C, n, g, act_order, x_kind="outlier", seed=0, reps=
     ms_step = (time.perf_counter() - t0) * 1e3 / reps
     assert not last[0].has_hessian_issues()
     del last
+    if PLAIN[0]:
+        return {"linear": name, "R": R, "C": C, "tokens": n, "group_size": g, "act_order": bool(act_order),
+                "ms_hessian_to_packed": round(ms_step, 3), "whole_steps_run": reps + 1, "roofline": None}
     hs = [make() for _ in range(reps)]
     for h in hs:
         h.update(X)
@@ -556,13 +566,15 @@ def config2_run(dev, cpu, reps=5):
     return leg
 
 
-def config4_run(dev, cpu, reps=3, cpu_full=False):
+def config4_run(dev, cpu, reps=3, cpu_full=False, only=None):
     """Config 4: the five MLA attention linears, 16384 tokens per input width, one at a time."""
     legs = {}
     for i, (name, (R, C)) in enumerate(CONFIG4_SHAPES.items()):
+        if only and name != only:
+            continue
         legs[name] = linear_leg(dev, name, R, C, 16384, 128, False, "outlier", seed=40 + i, reps=reps,
                                 profile_key="config4_hbm_traffic")
-    if cpu:
+    if cpu and "o_proj" in legs:
         # one bounded sample: o_proj, the linear that decides the block's attention part (16384^2 Hessian)
         Cs = 16384 if cpu_full else 4096
         legs["o_proj"]["cpu_baseline"] = cpu_linear_sample(7168, 16384, 16384, 128, False, "outlier", 512 if cpu_full else 2048,
@@ -570,24 +582,28 @@ def config4_run(dev, cpu, reps=3, cpu_full=False):
     return legs
 
 
-def config5_run(dev, cpu, reps=2, groups=(128, 64, 32), cpu_full=False):
+def config5_run(dev, cpu, reps=2, groups=(128, 64, 32), cpu_full=False, only=None):
     """Config 5: dense MLP with act-order, gate/up 18432x7168 and down 7168x18432, 65536 tokens, g in {128, 64, 32}."""
     legs = {}
     for g in groups:
-        legs[f"gate_up_g{g}"] = linear_leg(dev, f"gate_up g{g}", 18432, 7168, 65536, g, True, "outlier", seed=50, reps=reps,
-                                           profile_key="config5_hbm_traffic")
-        legs[f"down_g{g}"] = linear_leg(dev, f"down g{g}", 7168, 18432, 65536, g, True, "outlier", seed=51, reps=reps,
-                                        profile_key="config5_hbm_traffic")
-    if cpu:
+        if not only or only == f"gate_up_g{g}":
+            legs[f"gate_up_g{g}"] = linear_leg(dev, f"gate_up g{g}", 18432, 7168, 65536, g, True, "outlier", seed=50,
+                                               reps=reps, profile_key="config5_hbm_traffic")
+        if not only or only == f"down_g{g}":
+            legs[f"down_g{g}"] = linear_leg(dev, f"down g{g}", 7168, 18432, 65536, g, True, "outlier", seed=51, reps=reps,
+                                            profile_key="config5_hbm_traffic")
+    if cpu and f"down_g{groups[0]}" in legs:
         Cs = 18432 if cpu_full else 4096
         legs[f"down_g{groups[0]}"]["cpu_baseline"] = cpu_linear_sample(7168, 18432, 65536, groups[0], True, "outlier",
                                                                        256 if cpu_full else 2048, Cs, 1024 if cpu_full else 4096)
     return legs
 
 
-def _leg_line(metric, workload, legs, head):
+def _leg_line(metric, workload, legs, head=None):
     """One JSON line for a workload made of lone linears: value = linears/s over all of them, roofline and cpu_baseline
     of the linear `head` (the one the configuration is there to stress)."""
+    if head is None:
+        legs, head = legs
     total_ms = sum(l["ms_hessian_to_packed"] for l in legs.values())
     line = {
         "metric": metric, "value": round(len(legs) * 1000.0 / total_ms, 3), "unit": "linears/s", "n_gpus": 1,
@@ -608,21 +624,25 @@ def other_config_main(args):
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    cpu = not args.no_cpu_baseline
+    cpu = not args.no_cpu_baseline and not args.plain
+    PLAIN[0] = bool(args.plain)
+    rp = lambda d: args.reps if args.reps > 0 else d
     if args.workload == "config2":
-        leg = config2_run(dev, cpu)
+        leg = config2_run(dev, cpu, reps=rp(5))
         _leg_line("GPTQ linears/sec (7168x2048 expert down_proj, g128, packed)",
                   "config 2: expert down_proj 7168x2048 bf16, 65536 SwiGLU calibration tokens, 4-bit sym g128, packed int32 "
                   "words + bf16 scales; one linear per call", {"down_proj": leg}, "down_proj")
     elif args.workload == "config4":
         _leg_line("GPTQ linears/sec (MLA attention linears, g128)",
                   "config 4: q_a 1536x7168, q_b 24576x1536, kv_a 576x7168, kv_b 32768x512, o_proj 7168x16384, 16384 tokens per "
-                  "input width, 4-bit sym g128; one linear per call", config4_run(dev, cpu, cpu_full=True), "o_proj")
+                  "input width, 4-bit sym g128; one linear per call",
+                  (lambda legs: (legs, "o_proj" if "o_proj" in legs else next(iter(legs))))(
+                      config4_run(dev, cpu, reps=rp(3), cpu_full=True, only=args.only)))
     else:
-        legs = config5_run(dev, cpu, cpu_full=True)
+        legs = config5_run(dev, cpu, reps=rp(2), cpu_full=True, only=args.only)
         _leg_line("GPTQ linears/sec (dense MLP with act-order, g128/64/32)",
                   "config 5: gate/up 18432x7168 and down 7168x18432, 65536 tokens, act-order, 4-bit sym, group 128, 64 and 32; "
-                  "one linear per call", legs, "down_g128")
+                  "one linear per call", (legs, "down_g128" if "down_g128" in legs else next(iter(legs))))
 
 
 def main():
