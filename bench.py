@@ -350,8 +350,8 @@ def moe_layer_run(args, with_cpu_oracle=True):
                     "hessian": "the GPU's (same matrix on both sides)",
                     "tokens": n_tok,
                     # experts with fewer tokens than input channels have a singular Hessian held up by damping alone;
-                    # the test suite gates those at the oracle's own measured floor minus 0.1% instead of 99.9%
-                    "gate": 0.999 if n_tok >= w.shape[1] else "relaxed: oracle-against-itself floor - 0.001 (tests/test_gpu_moe_layer.py)",
+                    # the test suite gates those at the oracle's own measured floor minus 0.2% instead of 99.9%
+                    "gate": 0.999 if n_tok >= w.shape[1] else "relaxed: oracle-against-itself floor - 0.002 (tests/test_gpu_moe_layer.py)",
                     "scales_equal": bool(torch.equal(res.scales[f"{e}.{proj}"].cpu(), ref["scale"])),
                 }
         out["parity_vs_cpu_oracle"] = par
@@ -453,12 +453,22 @@ def syrk_main(args):
         H = torch.zeros(C, C, device=dev)
         alg = n * C * (C + 1)
         t_own = timed(lambda: ops.hessian_syrk_(H, X, 0.0, 2.0 / n, mirror=False))
+        Xp = ops.pack_tokens(X)
+        t_pack = timed(lambda: ops.pack_tokens(X))
+        Hp = torch.zeros(C, C, device=dev)
+        t_packed = timed(lambda: ops.hessian_syrk_packed_(Hp, Xp, 0.0, 2.0 / n, mirror=False))
+        same = bool(torch.equal(torch.triu(Hp), torch.triu(H)))
+        rel = ((torch.triu(Hp) - torch.triu(H)).norm() / torch.triu(H).norm()).item()
+        del Xp, Hp
         t_lib = timed(lambda: X.t() @ X)
         Xt = X.t().contiguous()
         t_lib_t = timed(lambda: Xt @ Xt.t())
         out[f"n={n} C={C}"] = {
             "mq_hessian_syrk_ms": round(t_own, 4), "algorithmic_tflops": round(alg / t_own / 1e9, 1),
             "frac_bf16_peak": round(alg / t_own / 1e9 / PEAK_BF16_MFMA, 4),
+            "mq_hessian_syrk_packed_ms": round(t_packed, 4), "packed_algorithmic_tflops": round(alg / t_packed / 1e9, 1),
+            "mq_pack_tokens_ms": round(t_pack, 4), "pack_gbps": round(4.0 * n * C / t_pack / 1e6, 1),
+            "packed_equals_token_major_bits": same, "packed_vs_token_major_rel_diff": rel,
             "vendor_gemm_same_layout_ms": round(t_lib, 4),
             "vendor_gemm_same_layout_executed_tflops": round(2.0 * n * C * C / t_lib / 1e9, 1),
             "vendor_gemm_pretransposed_ms": round(t_lib_t, 4),

@@ -69,6 +69,26 @@ int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const long* ldh, c
                                  const int* n, int C, const float* beta, const float* alpha, int mirror, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
+/* The same accumulation on tokens that were copied anyway and therefore laid out for the matrix cores by the copy
+ * (replaces the same src/gptq.py:97-103 product; the copies it rides on are the per-expert token gather of the block
+ * forward, quant.py:280-281, and the output of the SiLU product that feeds down_proj, mq_swiglu_packed below):
+ *   packed layout  Xp[o][c][j] = X[8 o + j][c]:  o = token octet, c = channel padded with zeros to a multiple of 256,
+ *   j = 0..7; tokens padded with zeros to a multiple of 128; mq_packed_tokens_bytes(n, C) bytes, 16-byte aligned.
+ *   mq_pack_tokens writes it from token-major 16-bit X (C and ldx multiples of 8, 16-byte aligned); rows != NULL
+ *   (device array of n int64 row indices) gathers X[rows[t]] in the same pass; Xg != NULL also receives the gathered
+ *   rows token-major (n x C, ldg), for the GEMMs of the model's own forward.
+ *   mq_hessian_syrk_packed reads it: H as in mq_hessian_syrk, n >= 1 real tokens, workspace of
+ *   mq_hessian_syrk_packed_workspace_bytes(n, C) bytes.  mq_hessian_syrk_packed_grouped: `groups` problems of one
+ *   width in one call (host arrays as in mq_hessian_syrk_grouped; no workspace). */
+size_t mq_packed_tokens_bytes(int n, int C);
+int mq_pack_tokens(const void* X, int x_dtype, long ldx, const long* rows, int n, int C, void* Xp, void* Xg, long ldg,
+                   void* stream);
+size_t mq_hessian_syrk_packed_workspace_bytes(int n, int C);
+int mq_hessian_syrk_packed(float* H, long ldh, const void* Xp, int x_dtype, int n, int C, float beta, float alpha,
+                           int mirror, void* workspace, size_t workspace_bytes, void* stream);
+int mq_hessian_syrk_packed_grouped(int groups, float* const* H, const long* ldh, const void* const* Xp, int x_dtype,
+                                   const int* n, int C, const float* beta, const float* alpha, int mirror, void* stream);
+
 /* lower triangle <- transpose of the upper triangle (what mirror != 0 does after the accumulation; exported so
  * that a caller accumulating many batches can mirror once at the end). */
 int mq_symmetrize_upper(float* H, long ldh, int C, void* stream);
@@ -282,6 +302,10 @@ int mq_dequant_fp8_block(const uint8_t* W, long ldw, int R, int C, const float* 
  * stacked weights), both roundings to `dtype` (MQ_DT_BF16 / MQ_DT_F16) as the chained torch ops round.
  *   I % 8 == 0, 16-byte aligned rows; out : n x I (ldo). */
 int mq_swiglu(const void* GU, long ldg, int n, int I, int dtype, void* out, long ldo, void* stream);
+/* The same product (same roundings) written straight into the packed-token layout mq_hessian_syrk_packed reads
+ * (mq_packed_tokens_bytes(n, I) bytes): its only reader is the down projection's Hessian.  G, U: the gate and the up
+ * projection's outputs, n x I each (ldg, ldu) -- two matrices or the two halves of one stacked GEMM output. */
+int mq_swiglu_packed(const void* G, long ldg, const void* U, long ldu, int n, int I, int dtype, void* out, void* stream);
 
 #ifdef __cplusplus
 }

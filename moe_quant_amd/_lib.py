@@ -21,6 +21,11 @@ SIGNATURES = {
     "mq_hessian_syrk_grouped_workspace_bytes": (_sz, [_i, _vp, _i]),
     "mq_hessian_syrk_grouped": (_i, [_i, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _i, _vp, _sz, _vp]),
     "mq_hessian_syrk_bf16_grouped": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _sz, _vp]),
+    "mq_packed_tokens_bytes": (_sz, [_i, _i]),
+    "mq_pack_tokens": (_i, [_vp, _i, _l, _vp, _i, _i, _vp, _vp, _l, _vp]),
+    "mq_hessian_syrk_packed_workspace_bytes": (_sz, [_i, _i]),
+    "mq_hessian_syrk_packed": (_i, [_vp, _l, _vp, _i, _i, _i, _f, _f, _i, _vp, _sz, _vp]),
+    "mq_hessian_syrk_packed_grouped": (_i, [_i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _vp]),
     "mq_symmetrize_upper": (_i, [_vp, _l, _i, _vp]),
     "mq_hessian_prestep": (_i, [_vp, _l, _i, _i, _vp, _vp, _vp]),
     "mq_permute_symmetric": (_i, [_vp, _l, _vp, _vp, _l, _i, _vp]),
@@ -47,6 +52,7 @@ SIGNATURES = {
     "mq_pack_from_qt": (_i, [_vp, _i, _i, _vp, _vp, _l, _vp]),
     "mq_dequant_fp8_block": (_i, [_vp, _l, _i, _i, _vp, _l, _i, _vp, _l, _vp]),
     "mq_swiglu": (_i, [_vp, _l, _i, _i, _i, _vp, _l, _vp]),
+    "mq_swiglu_packed": (_i, [_vp, _l, _vp, _l, _i, _i, _i, _vp, _vp]),
     "mq_gemm_f32": (_i, [_vp, _l, _l, _vp, _l, _l, _vp, _l, _i, _i, _i, _f, _f, _i, _i, _vp]),
 }
 

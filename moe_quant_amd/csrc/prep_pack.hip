@@ -377,14 +377,7 @@ __global__ __launch_bounds__(256) void dequant_fp8_kernel(const uint8_t* __restr
 // SwiGLU product of an expert: out[r, j] = round(round(silu(GU[r, j])) * GU[r, I + j]) for 16-bit GU (n x 2I: the gate
 // projection's outputs, then the up projection's), both roundings to the tensors' own type as the chained torch ops
 // `silu(g) * u` round.  Eight columns per thread, 16-byte accesses.
-__global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ GU, long ldg, int n, int I, int dt,
-                                                     uint16_t* __restrict__ out, long ldo) {
-  const int chunks = I / 8;
-  const long item = (long)blockIdx.x * 256 + threadIdx.x;
-  if (item >= (long)n * chunks) return;
-  const int r = (int)(item / chunks), c0 = (int)(item - (long)r * chunks) * 8;
-  const uint4 gv = *reinterpret_cast<const uint4*>(GU + (long)r * ldg + c0);
-  const uint4 uv = *reinterpret_cast<const uint4*>(GU + (long)r * ldg + I + c0);
+__device__ __forceinline__ uint4 swiglu8(const uint4 gv, const uint4 uv, int dt) {
   const uint32_t g[4] = {gv.x, gv.y, gv.z, gv.w}, u[4] = {uv.x, uv.y, uv.z, uv.w};
   uint32_t o[4];
 #pragma unroll
@@ -401,7 +394,49 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict_
     }
     o[k] = w;
   }
-  *reinterpret_cast<uint4*>(out + (long)r * ldo + c0) = make_uint4(o[0], o[1], o[2], o[3]);
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(const uint16_t* __restrict__ GU, long ldg, int n, int I, int dt,
+                                                     uint16_t* __restrict__ out, long ldo) {
+  const int chunks = I / 8;
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;
+  if (item >= (long)n * chunks) return;
+  const int r = (int)(item / chunks), c0 = (int)(item - (long)r * chunks) * 8;
+  const uint4 gv = *reinterpret_cast<const uint4*>(GU + (long)r * ldg + c0);
+  const uint4 uv = *reinterpret_cast<const uint4*>(GU + (long)r * ldg + I + c0);
+  *reinterpret_cast<uint4*>(out + (long)r * ldo + c0) = swiglu8(gv, uv, dt);
+}
+
+// The same product written in the packed-token layout the Hessian kernel reads (out[o][c][j] = value of token 8 o + j,
+// channel c; channels padded with zeros to Ip, tokens to a whole octet grid): the product's only reader is the down
+// projection's Hessian, so it never exists token-major.  G and U: the gate and the up projection's outputs, n x I each
+// (two matrices, or the two halves of one stacked GEMM output).  One thread per (token octet, channel octet).
+__global__ __launch_bounds__(256) void swiglu_packed_kernel(const uint16_t* __restrict__ G, long ldg,
+                                                            const uint16_t* __restrict__ U, long ldu, int n, int I, int Ip,
+                                                            int dt, uint16_t* __restrict__ out) {
+  const int o = blockIdx.y;
+  const int c8 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c8 >= Ip) return;
+  uint4 r[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int t = 8 * o + j;
+    r[j] = make_uint4(0, 0, 0, 0);
+    if (t < n && c8 < I)
+      r[j] = swiglu8(*reinterpret_cast<const uint4*>(G + (long)t * ldg + c8), *reinterpret_cast<const uint4*>(U + (long)t * ldu + c8), dt);
+  }
+  uint4* dst = reinterpret_cast<uint4*>(out + ((long)o * Ip + c8) * 8);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {  // word k of a row holds channels 2k (low half) and 2k+1 (high half)
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = k == 0 ? r[j].x : (k == 1 ? r[j].y : (k == 2 ? r[j].z : r[j].w));
+    dst[2 * k] = make_uint4((w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16), (w[4] & 0xffffu) | (w[5] << 16),
+                            (w[6] & 0xffffu) | (w[7] << 16));
+    dst[2 * k + 1] = make_uint4((w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
+                                (w[4] >> 16) | (w[5] & 0xffff0000u), (w[6] >> 16) | (w[7] & 0xffff0000u));
+  }
 }
 
 }  // namespace
@@ -414,6 +449,18 @@ extern "C" int mq_swiglu(const void* GU, long ldg, int n, int I, int dtype, void
   const long items = (long)n * (I / 8);
   hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                      (const uint16_t*)GU, ldg, n, I, dtype, (uint16_t*)out, ldo);
+  return mq_check_launch();
+}
+
+extern "C" int mq_swiglu_packed(const void* G, long ldg, const void* U, long ldu, int n, int I, int dtype, void* out,
+                                void* stream) {
+  if (n < 0 || I <= 0 || (I & 7) || ldg < I || ldu < I || (ldg & 7) || (ldu & 7)) return MQ_ERR_ARG;
+  if (dtype != DT_BF16 && dtype != DT_F16) return MQ_ERR_ARG;
+  if (n == 0) return MQ_OK;
+  if (!G || !U || !out || ((uintptr_t)G & 15) || ((uintptr_t)U & 15) || ((uintptr_t)out & 15)) return MQ_ERR_ARG;
+  const int Ip = (I + 255) / 256 * 256, octets = (n + 127) / 128 * 16;  // the packed layout's padding
+  hipLaunchKernelGGL(swiglu_packed_kernel, dim3((Ip / 8 + 255) / 256, octets), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)G, ldg, (const uint16_t*)U, ldu, n, I, Ip, dtype, (uint16_t*)out);
   return mq_check_launch();
 }
 

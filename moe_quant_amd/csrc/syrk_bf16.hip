@@ -13,6 +13,7 @@
 // partial tiles go to a caller-provided workspace and are reduced in a fixed order (deterministic).
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -536,6 +537,202 @@ __global__ __launch_bounds__(256) void symmetrize_kernel(float* __restrict__ H, 
   }
 }
 
+// =============================================================================================
+// Packed tokens.  The matrix cores want, per lane, eight consecutive tokens of one channel; token-major X has them
+// 2*ldx bytes apart, which is what the transposing LDS reads above are for.  Where the tokens are copied anyway (the
+// routed tokens of an expert are gathered; the output of the SiLU product is written by this library) the copy can
+// be laid out for the matrix cores instead:
+//     Xp[o][c][j] = X[8 o + j][c],   o = token octet, c = channel (padded to a multiple of 256), j = 0..7,
+// tokens padded with zeros to a multiple of 32.  A lane's operand fragment is then one aligned 16-byte cell, a
+// direct load moves 64 cells = 1 KB of contiguous memory to 1 KB of contiguous LDS, and fragments come out of LDS
+// with plain 16-byte reads (ds_read_b128, conflict-free: 16 lanes read 256 contiguous bytes).
+// Workgroup = eight wavefronts of 128x64 on a 256x256 tile, two per SIMD, as in the kernel above.  Stage = 32 tokens x
+// 512 channels = 32 KB ([token octet][channel][8 tokens]); four stages in LDS.  The loop is software-pipelined by hand
+// and its instruction order pinned: per 16-token step, eight matrix instructions with the next step's six fragment
+// reads and two direct loads of a later stage dealt between them; one barrier per stage, placed between the stage's two
+// steps, so that the fragments of the next stage's first step are fetched while the second step's products run.  Step A
+// of stage kt issues the second half of stage kt+3 (into the buffer of stage kt-1, free since that stage's barrier),
+// step B the first half of stage kt+4 (into the buffer of stage kt itself, which nobody reads after this stage's
+// barrier): three and a half stages in flight.  Loads past the last stage are not branched around: they fetch the last
+// stage again into a fifth, unread LDS area, which keeps the loop one basic block and the load counter's arithmetic
+// uniform.
+// Timing experiments on this loop (65536 tokens x 7168 channels; results discarded): no direct loads in the loop 1.34
+// PFLOP/s, loads that always hit the same L2-resident cells 1.22, no fragment reads 1.15, nothing but the matrix
+// instructions 1.43 -- the rate this chip sustains on dense bf16 products under its power limit with these tile
+// counts -- against 1.03-1.10 for the kernel as it is (the token-major kernel above: 0.93-0.98).
+// =============================================================================================
+constexpr int PK_PLANE = 512 * 16;            // bytes of one token octet of a stage
+constexpr int PK_STAGE = 4 * PK_PLANE;        // 32 KB
+constexpr int PK_NST = 4;
+constexpr size_t PK_SMEM = (size_t)(PK_NST + 1) * PK_STAGE;  // + the dump area: 160 KB, all the LDS of a CU
+
+static inline int pk_pad_tokens(int n) { return (n + 127) / 128 * 128; }
+static inline int pk_pad_channels(int C) { return (C + 255) / 256 * 256; }
+
+template <bool F16>
+__device__ __forceinline__ void syrk_packed_tile(float* __restrict__ H, long ldh, const uint16_t* __restrict__ Xp, int n_pad,
+                                                  int Cp, int C, float alpha, float beta, SyrkPlan pl, float* __restrict__ ws,
+                                                  int bid, int yrow, unsigned char* smem) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int split = max(yrow - 1, 0);
+  const bool partial = yrow > 0;
+  if (bid >= (partial ? pl.ntail : pl.head)) return;
+  const int L = partial ? pl.head + bid : xcd_remap(bid, pl.head);
+  int tm, tn;
+  blocked_tri_decode(L, Cp / T2, tm, tn);
+  tm = __builtin_amdgcn_readfirstlane(tm);
+  tn = __builtin_amdgcn_readfirstlane(tn);
+  const int m0 = tm * T2, n0 = tn * T2;
+  const int tbeg = partial ? __builtin_amdgcn_readfirstlane(min(n_pad, split * pl.tps)) : 0;
+  const int tend = partial ? min(n_pad, tbeg + pl.tps) : n_pad;
+  const int nk = (tend - tbeg) / 32;
+  const int s0 = tbeg / 32;
+  const unsigned smem_lds = __builtin_amdgcn_readfirstlane(
+      (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem);
+  const unsigned lane_off = 16u * (unsigned)lane;
+  floatx16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  if (nk > 0) {
+    // direct load q (0..3) of stage s: token octet wave/2 of the stage; even wavefronts fetch the row tile's four
+    // 64-channel groups, odd ones the column tile's
+    const int oct = wave >> 1, side = wave & 1;
+    auto issue = [&](int s, int q) {
+      const int src = min(s, nk - 1);
+      const long cell = ((long)(s0 + src) * 4 + oct) * Cp + (side ? n0 : m0) + 64 * q;
+      const unsigned dst = smem_lds + (unsigned)((s < nk ? s % PK_NST : PK_NST) * PK_STAGE + oct * PK_PLANE + (4 * side + q) * 1024);
+      dma16(Xp + cell * 8, lane_off, dst);
+    };
+#pragma unroll
+    for (int s = 0; s < PK_NST - 1; ++s)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) issue(s, q);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) issue(PK_NST - 1, q);
+    const int lr = lane & 31, lk = lane >> 5;
+    const int a_off = lk * PK_PLANE + (wm * 128 + lr) * 16;
+    const int b_off = lk * PK_PLANE + (256 + wn * 64 + lr) * 16;
+    bf16x8n fa0[4], fb0[2], fa1[4], fb1[2];
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | 10);  // stage 0 landed: at most the 10 loads of stages 1, 2, 3 in flight
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8n*>(smem + a_off + i * 512);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) fb0[j] = *reinterpret_cast<const bf16x8n*>(smem + b_off + j * 512);
+#pragma unroll 1
+    for (int kt = 0; kt < nk; ++kt) {
+      const unsigned char* stg = smem + (kt % PK_NST) * PK_STAGE;
+      const unsigned char* nxt = smem + ((kt + 1) % PK_NST) * PK_STAGE;
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        acc[m >> 1][m & 1] = mfma16<F16>(fa0[m >> 1], fb0[m & 1], acc[m >> 1][m & 1]);
+        if (m < 4) fa1[m] = *reinterpret_cast<const bf16x8n*>(stg + 2 * PK_PLANE + a_off + m * 512);
+        else if (m < 6) fb1[m - 4] = *reinterpret_cast<const bf16x8n*>(stg + 2 * PK_PLANE + b_off + (m - 4) * 512);
+        else issue(kt + PK_NST - 1, 2 + (m - 6));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0x0070 | 8);  // stage kt+1 landed: at most the 8 loads of stages kt+2, kt+3 in flight
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        acc[m >> 1][m & 1] = mfma16<F16>(fa1[m >> 1], fb1[m & 1], acc[m >> 1][m & 1]);
+        if (m < 4) fa0[m] = *reinterpret_cast<const bf16x8n*>(nxt + a_off + m * 512);
+        else if (m < 6) fb0[m - 4] = *reinterpret_cast<const bf16x8n*>(nxt + b_off + (m - 4) * 512);
+        else issue(kt + PK_NST, m - 6);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);
+  }
+  const int lr = lane & 31, lk = lane >> 5;
+  float* out = partial ? ws + ((long)split * pl.ntail + (L - pl.head)) * (T2 * T2) : H;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = wn * 64 + j * 32 + lr;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+        if (partial) {
+          out[r * T2 + c] = acc[i][j][v];
+        } else if (m0 + r < C && n0 + c < C) {
+          float* q = H + (long)(m0 + r) * ldh + n0 + c;
+          float val = alpha * acc[i][j][v];
+          if (beta != 0.f) val = fmaf(beta, *q, val);
+          *q = val;
+        }
+      }
+    }
+}
+template <bool F16>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_packed_kernel(
+    float* __restrict__ H, long ldh, const uint16_t* __restrict__ Xp, int n_pad, int Cp, int C, float alpha, float beta,
+    SyrkPlan pl, float* __restrict__ ws) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  syrk_packed_tile<F16>(H, ldh, Xp, n_pad, Cp, C, alpha, beta, pl, ws, blockIdx.x, blockIdx.y, smem);
+}
+
+// Several independent accumulations on packed tokens (one Hessian each, same C) in one launch: blockIdx.y picks the
+// problem, every workgroup runs the whole token range of its tile (no partial tiles, no workspace).
+struct SyrkPackedTable {
+  float* H[SYRK_MAX_GROUP];
+  const uint16_t* Xp[SYRK_MAX_GROUP];
+  long ldh[SYRK_MAX_GROUP];
+  int n_pad[SYRK_MAX_GROUP];
+  float alpha[SYRK_MAX_GROUP], beta[SYRK_MAX_GROUP];
+};
+template <bool F16>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_packed_grouped_kernel(SyrkPackedTable t,
+                                                                                                              int Cp, int C,
+                                                                                                              int ntri) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int z = blockIdx.y;
+  syrk_packed_tile<F16>(t.H[z], t.ldh[z], t.Xp[z], t.n_pad[z], Cp, C, t.alpha[z], t.beta[z], SyrkPlan{ntri, ntri, 0, 1, 0},
+                        nullptr, blockIdx.x, 0, smem);
+}
+
+// X (n x C, 16-bit, row pitch ldx; rows != nullptr: row t of the input is X[rows[t]]) -> the packed layout above and,
+// when Xg != nullptr, the gathered rows once more in token-major order (n x C, row pitch ldg: what a GEMM of the
+// model's forward wants).  A wavefront handles one token octet x 64 channels: lane (token j = lane % 8, channel octet
+// q = lane / 8) loads 16 bytes (eight rows x 128 bytes per instruction), the 8 x 64 patch is turned in LDS, and lane c
+// stores the finished cell of channel c: 1 KB of contiguous memory per store instruction.  Tokens past n and channels
+// past C are zeros.
+__global__ __launch_bounds__(256) void pack_tokens_kernel(const uint16_t* __restrict__ X, long ldx, const long* __restrict__ rows,
+                                                         int n, int C, int Cp, uint16_t* __restrict__ Xp,
+                                                         uint16_t* __restrict__ Xg, long ldg) {
+  constexpr int PITCH = 64 + 8;  // 16-bit elements per LDS row: 144 bytes, so the eight rows of a column start in eight banks
+  __shared__ __attribute__((aligned(16))) uint16_t patch[4][8 * PITCH];
+  const int o = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c0 = (blockIdx.x * 4 + wave) * 64;
+  const int j = lane & 7, q = lane >> 3;
+  const int t = 8 * o + j, c8 = c0 + 8 * q;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (t < n && c8 < C) {
+    const long row = rows ? rows[t] : (long)t;
+    v = *reinterpret_cast<const uint4*>(X + row * ldx + c8);
+    if (Xg) *reinterpret_cast<uint4*>(Xg + (long)t * ldg + c8) = v;
+  }
+  uint16_t* p = patch[wave];
+  *reinterpret_cast<uint4*>(p + j * PITCH + 8 * q) = v;
+  __syncthreads();  // (every wavefront of the grid has work: Cp is a multiple of the 256 channels a workgroup covers)
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+    w[k] = (uint32_t)p[(2 * k) * PITCH + lane] | ((uint32_t)p[(2 * k + 1) * PITCH + lane] << 16);
+  *reinterpret_cast<uint4*>(Xp + ((long)o * Cp + c0 + lane) * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 constexpr int NCU = 256;  // workgroups the large-tile kernel keeps resident (one per CU)
 
 SyrkPlan plan_big(int n, int C) {
@@ -602,13 +799,36 @@ void pick_split(int n, int C, int& ntri, int& splits, int& tps) {
 
 }  // namespace
 
+extern "C" size_t mq_packed_tokens_bytes(int n, int C);
+extern "C" int mq_pack_tokens(const void* X, int x_dtype, long ldx, const long* rows, int n, int C, void* Xp, void* Xg,
+                              long ldg, void* stream);
+extern "C" size_t mq_hessian_syrk_packed_workspace_bytes(int n, int C);
+extern "C" int mq_hessian_syrk_packed(float* H, long ldh, const void* Xp, int x_dtype, int n, int C, float beta, float alpha,
+                                      int mirror, void* workspace, size_t workspace_bytes, void* stream);
+extern "C" int mq_hessian_syrk_packed_grouped(int groups, float* const* H, const long* ldh, const void* const* Xp, int x_dtype,
+                                              const int* n, int C, const float* beta, const float* alpha, int mirror,
+                                              void* stream);
+
+// Wide Hessians with many tokens: one pass re-lays the token-major activations out for the matrix cores (6 TB/s, a
+// tenth of the product's time) and the product runs on the packed-token kernel: 0.44 against 0.52 ms for 8192 tokens
+// x 7168 channels, 0.385 against 0.44 ms per Hessian in calls of eight.  Narrow ones (2048 channels) and short token
+// runs gain nothing and stay on the token-major kernel.
+static bool route_packed(const void* X, long ldx, int n, int C) {
+  return n >= 4096 && C >= 4096 && (C % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
+}
+static size_t packed_route_ws_bytes(int n, int C) {
+  return n >= 4096 && C >= 4096 ? mq_packed_tokens_bytes(n, C) + mq_hessian_syrk_packed_workspace_bytes(n, C) : 0;
+}
+
 extern "C" size_t mq_hessian_syrk_workspace_bytes(int n, int C) {
   if (n <= 0 || C <= 0) return 0;
   int ntri, splits, tps;
   pick_split(n, C, ntri, splits, tps);
   const size_t small = splits > 1 ? (size_t)splits * ntri * T * T * sizeof(float) : 0;
   const size_t big = plan_big_ws_bytes(plan_big(n, C));
-  return small > big ? small : big;  // either kernel may be chosen, depending on alignment
+  const size_t packed = packed_route_ws_bytes(n, C);
+  const size_t m = small > big ? small : big;  // any of the kernels may be chosen, depending on alignment
+  return m > packed ? m : packed;
 }
 
 extern "C" int mq_symmetrize_upper(float* H, long ldh, int C, void* stream) {
@@ -653,6 +873,14 @@ extern "C" int mq_hessian_syrk(float* H, long ldh, const void* X, int x_dtype, l
                               (int)SMEM_BYTES);
     (void)hipFuncSetAttribute((const void*)syrk_reduce_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES);
   });
+  if (route_packed(X, ldx, n, C)) {
+    const size_t pb = mq_packed_tokens_bytes(n, C), need = pb + mq_hessian_syrk_packed_workspace_bytes(n, C);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return MQ_ERR_WORKSPACE;
+    const int rc = mq_pack_tokens(X, x_dtype, ldx, nullptr, n, C, workspace, nullptr, 0, stream);
+    if (rc != MQ_OK) return rc;
+    return mq_hessian_syrk_packed(H, ldh, workspace, x_dtype, n, C, beta, alpha, mirror, (char*)workspace + pb,
+                                  workspace_bytes - pb, stream);
+  }
   if (n > 0 && use_big(X, ldx, n, C)) {
     const SyrkPlan pl = plan_big(n, C);
     const size_t need = plan_big_ws_bytes(pl);
@@ -703,12 +931,13 @@ extern "C" int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx,
 // rows, fp32 tokens) make the whole call fall back to one plain call per problem, so the result never depends on
 // the path.
 extern "C" size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C) {
-  size_t need = 0;
+  size_t need = 0, packed = 0;
   for (int g = 0; g < groups; ++g) {
     const size_t w = mq_hessian_syrk_workspace_bytes(n[g], C);
     if (w > need) need = w;
+    packed += n[g] >= 4096 && C >= 4096 ? mq_packed_tokens_bytes(n[g], C) : 0;  // the packed route packs every problem first
   }
-  return need;
+  return need > packed ? need : packed;
 }
 
 extern "C" int mq_hessian_syrk_grouped(int groups, float* const* H, const long* ldh, const void* const* X, int x_dtype,
@@ -722,6 +951,23 @@ extern "C" int mq_hessian_syrk_grouped(int groups, float* const* H, const long* 
     if (n[g] <= 0 || !use_big(X[g], ldx[g], n[g], C)) fast = false;
   }
   hipStream_t st = (hipStream_t)stream;
+  bool packed = groups > 1 && x_dtype != MQ_DT_F32 && groups <= 64;
+  size_t pbytes = 0;
+  for (int g = 0; g < groups && packed; ++g) {
+    packed = route_packed(X[g], ldx[g], n[g], C);
+    pbytes += packed ? mq_packed_tokens_bytes(n[g], C) : 0;
+  }
+  if (packed && workspace && workspace_bytes >= pbytes && !((uintptr_t)workspace & 15)) {
+    const void* Xp[64];
+    char* w = (char*)workspace;
+    for (int g = 0; g < groups; ++g) {
+      const int rc = mq_pack_tokens(X[g], x_dtype, ldx[g], nullptr, n[g], C, w, nullptr, 0, stream);
+      if (rc != MQ_OK) return rc;
+      Xp[g] = w;
+      w += mq_packed_tokens_bytes(n[g], C);
+    }
+    return mq_hessian_syrk_packed_grouped(groups, H, ldh, Xp, x_dtype, n, C, beta, alpha, mirror, stream);
+  }
   if (!fast) {
     for (int g = 0; g < groups; ++g) {
       const int rc = mq_hessian_syrk(H[g], ldh[g], X[g], x_dtype, ldx[g], n[g], C, beta[g], alpha[g], mirror, workspace,
@@ -769,4 +1015,101 @@ extern "C" int mq_hessian_syrk_bf16_grouped(int groups, float* const* H, const l
                                             int mirror, void* workspace, size_t workspace_bytes, void* stream) {
   return mq_hessian_syrk_grouped(groups, H, ldh, X, MQ_DT_BF16, ldx, n, C, beta, alpha, mirror, workspace, workspace_bytes,
                                  stream);
+}
+
+// ---- packed tokens ------------------------------------------------------------------------------------------------
+extern "C" size_t mq_packed_tokens_bytes(int n, int C) {
+  if (n <= 0 || C <= 0) return 0;
+  return (size_t)pk_pad_tokens(n) * pk_pad_channels(C) * 2;
+}
+
+extern "C" int mq_pack_tokens(const void* X, int x_dtype, long ldx, const long* rows, int n, int C, void* Xp, void* Xg,
+                              long ldg, void* stream) {
+  if (n < 0 || C <= 0 || (n > 0 && (!X || !Xp || ldx < C))) return MQ_ERR_ARG;
+  if (x_dtype != MQ_DT_BF16 && x_dtype != MQ_DT_F16) return MQ_ERR_ARG;
+  if ((C & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)Xp & 15)) return MQ_ERR_ARG;  // 16-byte loads and cells
+  if (Xg && (ldg < C || (ldg & 7) || ((uintptr_t)Xg & 15))) return MQ_ERR_ARG;
+  if (n == 0) return MQ_OK;
+  const int Cp = pk_pad_channels(C), octets = pk_pad_tokens(n) / 8;
+  hipLaunchKernelGGL(pack_tokens_kernel, dim3(Cp / 256, octets), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)X, ldx, rows, n, C, Cp, (uint16_t*)Xp, (uint16_t*)Xg, ldg);
+  return mq_check_launch();
+}
+
+extern "C" size_t mq_hessian_syrk_packed_workspace_bytes(int n, int C) {
+  if (n <= 0 || C <= 0) return 0;
+  return plan_big_ws_bytes(plan_big(pk_pad_tokens(n), pk_pad_channels(C)));
+}
+
+extern "C" int mq_hessian_syrk_packed(float* H, long ldh, const void* Xp, int x_dtype, int n, int C, float beta, float alpha,
+                                      int mirror, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!H || C <= 0 || n <= 0 || ldh < C || !Xp || ((uintptr_t)Xp & 15)) return MQ_ERR_ARG;
+  if (x_dtype != MQ_DT_BF16 && x_dtype != MQ_DT_F16) return MQ_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)syrk_packed_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)PK_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_packed_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)PK_SMEM);
+  });
+  const int n_pad = pk_pad_tokens(n), Cp = pk_pad_channels(C);
+  const SyrkPlan pl = plan_big(n_pad, Cp);
+  const size_t need = plan_big_ws_bytes(pl);
+  if (need && (!workspace || workspace_bytes < need)) return MQ_ERR_WORKSPACE;
+  const dim3 grid(pl.head > pl.ntail ? pl.head : pl.ntail, pl.ntail ? 1 + pl.splits : 1);
+  if (x_dtype == MQ_DT_F16)
+    hipLaunchKernelGGL(syrk_packed_kernel<true>, grid, dim3(512), PK_SMEM, st, H, ldh, (const uint16_t*)Xp, n_pad, Cp, C, alpha,
+                       beta, pl, (float*)workspace);
+  else
+    hipLaunchKernelGGL(syrk_packed_kernel<false>, grid, dim3(512), PK_SMEM, st, H, ldh, (const uint16_t*)Xp, n_pad, Cp, C, alpha,
+                       beta, pl, (float*)workspace);
+  int rc = mq_check_launch();
+  if (rc != MQ_OK) return rc;
+  if (pl.ntail) {
+    hipLaunchKernelGGL(syrk_big_reduce_kernel, dim3(T2 * T2 / 4 / 256, pl.ntail), dim3(256), 0, st, H, ldh, C, alpha, beta, pl,
+                       (const float*)workspace);
+    if ((rc = mq_check_launch()) != MQ_OK) return rc;
+  }
+  return mirror ? mq_symmetrize_upper(H, ldh, C, stream) : MQ_OK;
+}
+
+// Host arrays of `groups` entries each; every problem n >= 1.  Up to 16 problems share a launch.
+extern "C" int mq_hessian_syrk_packed_grouped(int groups, float* const* H, const long* ldh, const void* const* Xp, int x_dtype,
+                                              const int* n, int C, const float* beta, const float* alpha, int mirror,
+                                              void* stream) {
+  if (groups < 0 || C <= 0 || (groups > 0 && (!H || !ldh || !Xp || !n || !beta || !alpha))) return MQ_ERR_ARG;
+  if (x_dtype != MQ_DT_BF16 && x_dtype != MQ_DT_F16) return MQ_ERR_ARG;
+  for (int g = 0; g < groups; ++g)
+    if (!H[g] || !Xp[g] || n[g] <= 0 || ldh[g] < C || ((uintptr_t)Xp[g] & 15)) return MQ_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    (void)hipFuncSetAttribute((const void*)syrk_packed_grouped_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)PK_SMEM);
+    (void)hipFuncSetAttribute((const void*)syrk_packed_grouped_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)PK_SMEM);
+  });
+  const int Cp = pk_pad_channels(C), tiles = Cp / T2, ntri = tiles * (tiles + 1) / 2;
+  for (int g0 = 0; g0 < groups; g0 += SYRK_MAX_GROUP) {
+    const int cnt = groups - g0 < SYRK_MAX_GROUP ? groups - g0 : SYRK_MAX_GROUP;
+    SyrkPackedTable t;
+    for (int i = 0; i < SYRK_MAX_GROUP; ++i) {
+      const int g = g0 + (i < cnt ? i : 0);
+      t.H[i] = H[g];
+      t.Xp[i] = (const uint16_t*)Xp[g];
+      t.ldh[i] = ldh[g];
+      t.n_pad[i] = pk_pad_tokens(n[g]);
+      t.alpha[i] = alpha[g];
+      t.beta[i] = beta[g];
+    }
+    if (x_dtype == MQ_DT_F16)
+      hipLaunchKernelGGL(syrk_packed_grouped_kernel<true>, dim3(ntri, cnt), dim3(512), PK_SMEM, st, t, Cp, C, ntri);
+    else
+      hipLaunchKernelGGL(syrk_packed_grouped_kernel<false>, dim3(ntri, cnt), dim3(512), PK_SMEM, st, t, Cp, C, ntri);
+    int rc = mq_check_launch();
+    if (rc != MQ_OK) return rc;
+    if (mirror)
+      for (int i = 0; i < cnt; ++i)
+        if ((rc = mq_symmetrize_upper(H[g0 + i], ldh[g0 + i], C, stream)) != MQ_OK) return rc;
+  }
+  return MQ_OK;
 }

@@ -136,7 +136,12 @@ class GPTQ:
 
     # ---- Hessian accumulation: src/gptq.py:73-105 ---------------------------------------------------
     @torch.no_grad()
-    def update(self, input: Tensor) -> None:
+    def update(self, input) -> None:
+        """`input`: the activations the forward hook delivers (..., C), or an `ops.PackedTokens` of them (the same
+        tokens in the layout the matrix cores read, for callers that copy the tokens anyway: ops.pack_tokens gathers
+        and re-lays them out in one pass, ops.swiglu_packed writes a down projection's inputs that way)."""
+        if isinstance(input, ops.PackedTokens):
+            return GPTQ.update_many([self], [input])
         input = input.reshape(-1, input.shape[-1])
         if input.dtype not in _ACT_DTYPES:
             raise TypeError(f"GPTQ.update takes bf16, fp16 or fp32 activations, got {input.dtype}")
@@ -168,23 +173,39 @@ class GPTQ:
         """`h.update(x)` for several handles of one input width with one library call (the experts of a block,
         whose hooks the reference serves one addmm_ at a time).  Same arithmetic per handle as `update`."""
         Hs, Xs, betas, alphas = [], [], [], []
+        inputs = list(inputs)
+        packed = bool(inputs) and isinstance(inputs[0], ops.PackedTokens)
+        if any(isinstance(x, ops.PackedTokens) != packed for x in inputs):
+            raise TypeError("update_many takes either tensors or PackedTokens, not a mix")
         for h, x in zip(handles, inputs):
-            x = x.reshape(-1, x.shape[-1])
-            if x.dtype not in _ACT_DTYPES:
-                raise TypeError(f"GPTQ.update takes bf16, fp16 or fp32 activations, got {x.dtype}")
-            if x.shape[0] == 0:
+            if packed:
+                if x.C != h.d_col:
+                    raise ValueError(f"packed tokens have {x.C} channels, the layer {h.d_col}")
+                n_x = x.n
+            else:
+                x = x.reshape(-1, x.shape[-1])
+                if x.dtype not in _ACT_DTYPES:
+                    raise TypeError(f"GPTQ.update takes bf16, fp16 or fp32 activations, got {x.dtype}")
+                n_x = x.shape[0]
+            if n_x == 0:
                 continue
             if h.H is None:
                 alloc = torch.empty if h.num_samples == 0 else torch.zeros  # beta = 0 below: nothing to clear
-                h.H = alloc((h.d_col, h.d_col), device=x.device, dtype=torch.float32)
-            n = x.shape[0]
+                h.H = alloc((h.d_col, h.d_col), device=(x.data if packed else x).device, dtype=torch.float32)
+            n = n_x
             Hs.append(h.H)
             Xs.append(x)
             betas.append(h.num_samples / (h.num_samples + n))
             alphas.append(2.0 / (h.num_samples + n))
             h.num_samples += n
             h._H_upper_only, h._H_clean = True, False
-        ops.hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror=False)
+        if packed:
+            if len(Hs) == 1:
+                ops.hessian_syrk_packed_(Hs[0], Xs[0], betas[0], alphas[0], mirror=False)
+            else:
+                ops.hessian_syrk_packed_grouped_(Hs, Xs, betas, alphas, mirror=False)
+        else:
+            ops.hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror=False)
 
     @property
     def tokens_collected(self) -> int:

@@ -111,24 +111,53 @@ def quantize_moe_layer(
     factor_calls_before = GPTQ.factor_calls
     group = max(1, group)
 
+    # Hessian products wait here until `group` of one width have come together (or the same handle comes again: two
+    # products into one H must not share a launch); then they run as one grouped library call.
+    pending = {"gate_up": [], "down": []}
+
+    def flush(kind):
+        for want_packed in (True, False):
+            part = [(h, p) for h, p in pending[kind] if isinstance(p, ops.PackedTokens) == want_packed]
+            if part:
+                GPTQ.update_many([h for h, _ in part], [p for _, p in part])
+        pending[kind].clear()
+
+    def enqueue(kind, h, tokens):
+        if any(h is q for q, _ in pending[kind]):
+            flush(kind)
+        pending[kind].append((h, tokens))
+        if len(pending[kind]) >= group:
+            flush(kind)
+
+    packable = x.dtype in (torch.bfloat16, torch.float16) and x.shape[1] % 8 == 0 and experts[0].gate.shape[0] % 8 == 0
+
     def collect_hessians(e):
-        """Hessians of expert e (gate and up share one, quant.py:258-277) from its routed tokens."""
+        """Hessians of expert e (gate and up share one, quant.py:258-277) from its routed tokens: one pass gathers the
+        expert's rows of x twice -- token-major for the two GEMMs of the expert's own forward (the model's matmuls,
+        rocBLAS/hipBLASLt through torch) and in the packed layout the Hessian kernel reads -- and the SiLU product is
+        written straight into that layout, its only reader being the down projection's Hessian."""
         g, u, d = handles[e]
         lo, hi = offsets[e], offsets[e + 1]
-        gate_up = None
         for s in range(lo, hi, max_rows_per_update):
             idx = rows[s : min(hi, s + max_rows_per_update)]
-            xe = x.index_select(0, idx)  # (n, C) bf16
-            g.update(xe)
-            # the expert's forward up to the down projection's input: one GEMM against the stacked gate/up weights
-            # (the model's own matmul, rocBLAS/hipBLASLt through torch), then the SwiGLU product in one pass
-            if gate_up is None:
-                gate_up = torch.cat([experts[e].gate, experts[e].up], dim=0)
-            a = ops.swiglu(xe @ gate_up.t())
-            d.update(a)
+            if packable and idx.numel() >= 256:
+                P, xe = ops.pack_tokens(x, idx, also_token_major=True)
+                enqueue("gate_up", g, P)
+                A = ops.swiglu_packed(xe @ experts[e].gate.t(), xe @ experts[e].up.t())
+                enqueue("down", d, A)
+                a = ops.unpack_tokens(A) if e in keep_codes else None
+            else:  # a handful of tokens: plain tensors
+                xe = x.index_select(0, idx)
+                enqueue("gate_up", g, xe)
+                a = ops.swiglu(torch.cat([xe @ experts[e].gate.t(), xe @ experts[e].up.t()], dim=1))
+                enqueue("down", d, a)
             if e in keep_codes:
                 prev = res.down_inputs.get(e)
                 res.down_inputs[e] = a if prev is None else torch.cat([prev, a])
+
+    def hessians_done():
+        flush("gate_up")
+        flush("down")
 
     def quantize_chunk(chunk):
         """Quantize + pack the three linears of every expert of the chunk (on the current stream)."""
@@ -176,6 +205,7 @@ def quantize_moe_layer(
         for ci, chunk in enumerate(chunks):
             for e in chunk:
                 collect_hessians(e)
+            hessians_done()
             ready = torch.cuda.Event()
             ready.record(main)
             lane = lanes[ci % len(lanes)]
@@ -188,6 +218,7 @@ def quantize_moe_layer(
         for chunk in chunks:
             for e in chunk:
                 collect_hessians(e)
+        hessians_done()
         ev1.record(main)
         sync()
         for s_ in lanes:

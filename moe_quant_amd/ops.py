@@ -111,6 +111,90 @@ def hessian_syrk_grouped_(Hs, Xs, betas, alphas, mirror: bool = True) -> None:
     check(rc, "mq_hessian_syrk_grouped")
 
 
+class PackedTokens:
+    """Activations laid out for the matrix cores: Xp[o][c][j] = X[8 o + j][c] (token octet o, channel c padded to a
+    multiple of 256, j = 0..7), tokens padded with zeros to a multiple of 32.  Made by `pack_tokens`, read by
+    `hessian_syrk_packed_`."""
+
+    def __init__(self, data: Tensor, n: int, C: int, dtype: torch.dtype):
+        self.data, self.n, self.C, self.dtype = data, n, C, dtype
+
+
+def pack_tokens(X: Tensor, rows: Optional[Tensor] = None, also_token_major: bool = False):
+    """X (m, C) bf16/fp16 -> PackedTokens of X (rows None) or of X[rows] (rows: int64 indices on the device; the
+    gather and the re-layout are one pass).  also_token_major: returns (PackedTokens, Xg) with Xg the gathered rows
+    once more as an ordinary (n, C) tensor, written by the same pass (for the GEMMs of the model's forward)."""
+    _dev(X, rows)
+    lib = _lib.load()
+    if X.dim() != 2 or X.dtype not in (torch.bfloat16, torch.float16) or X.stride(1) != 1:
+        raise ValueError("X must be (m, C) bf16/fp16 with unit column stride")
+    if rows is not None and (rows.dtype != torch.int64 or rows.dim() != 1 or not rows.is_contiguous()):
+        raise ValueError("rows must be a contiguous int64 vector")
+    C = X.shape[1]
+    n = X.shape[0] if rows is None else rows.numel()
+    nbytes = lib.mq_packed_tokens_bytes(n, C)
+    out = torch.empty(max(nbytes, 16) // 2, dtype=X.dtype, device=X.device)
+    Xg = torch.empty(n, C, dtype=X.dtype, device=X.device) if also_token_major else None
+    rc = lib.mq_pack_tokens(X.data_ptr(), _DT[X.dtype], X.stride(0), _p(rows), n, C, out.data_ptr(), _p(Xg), C, _stream(X))
+    check(rc, "mq_pack_tokens")
+    P = PackedTokens(out, n, C, X.dtype)
+    return (P, Xg) if also_token_major else P
+
+
+def unpack_tokens(P: PackedTokens) -> Tensor:
+    """PackedTokens -> the ordinary (n, C) tensor (a torch view/copy; for tests and debugging)."""
+    Cp = (P.C + 255) // 256 * 256
+    octets = (P.n + 127) // 128 * 16
+    return P.data[: octets * Cp * 8].view(octets, Cp, 8).permute(0, 2, 1).reshape(octets * 8, Cp)[: P.n, : P.C].contiguous()
+
+
+def hessian_syrk_packed_(H: Tensor, Xp: PackedTokens, beta: float, alpha: float, mirror: bool = True) -> Tensor:
+    """H <- beta*H + alpha*X^T X in place, X given as PackedTokens."""
+    _dev(H, Xp.data)
+    lib = _lib.load()
+    C = H.shape[0]
+    if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1 or Xp.C != C:
+        raise ValueError("H must be a (C,C) fp32 matrix with unit column stride, C the packed tokens' width")
+    if Xp.n <= 0:
+        if beta != 1.0:
+            H.mul_(beta)
+        return H
+    need = lib.mq_hessian_syrk_packed_workspace_bytes(Xp.n, C)
+    ws = _ws.get(H.device, need, "syrk") if need else None
+    rc = lib.mq_hessian_syrk_packed(H.data_ptr(), H.stride(0), Xp.data.data_ptr(), _DT[Xp.dtype], Xp.n, C, beta, alpha,
+                                    int(mirror), _p(ws), need, _stream(H))
+    check(rc, "mq_hessian_syrk_packed")
+    return H
+
+
+def hessian_syrk_packed_grouped_(Hs, Xps, betas, alphas, mirror: bool = True) -> None:
+    """hessian_syrk_packed_ for several Hessians of one width with one library call (every problem at least one token)."""
+    import ctypes as C_
+
+    lib = _lib.load()
+    k = len(Hs)
+    if not (len(Xps) == len(betas) == len(alphas) == k):
+        raise ValueError("Hs, Xps, betas, alphas must have the same length")
+    if k == 0:
+        return
+    _dev(*Hs, *[x.data for x in Xps])
+    C = Hs[0].shape[0]
+    dt = Xps[0].dtype
+    for H, X in zip(Hs, Xps):
+        if H.dtype != torch.float32 or H.shape != (C, C) or H.stride(1) != 1:
+            raise ValueError("every H must be a (C,C) fp32 matrix with unit column stride")
+        if X.C != C or X.dtype != dt or X.n <= 0:
+            raise ValueError("every packed X must have C channels, one dtype and at least one token")
+    ns = (C_.c_int * k)(*[x.n for x in Xps])
+    Hp = (C_.c_void_p * k)(*[h.data_ptr() for h in Hs])
+    Xp = (C_.c_void_p * k)(*[x.data.data_ptr() for x in Xps])
+    ldh = (C_.c_long * k)(*[h.stride(0) for h in Hs])
+    be = (C_.c_float * k)(*[float(b) for b in betas])
+    al = (C_.c_float * k)(*[float(a) for a in alphas])
+    rc = lib.mq_hessian_syrk_packed_grouped(k, Hp, ldh, Xp, _DT[dt], ns, C, be, al, int(mirror), _stream(Hs[0]))
+    check(rc, "mq_hessian_syrk_packed_grouped")
+
+
 def symmetrize_upper_(H: Tensor) -> Tensor:
     """Copies the upper triangle of H onto the lower one, in place."""
     _dev(H)
@@ -524,6 +608,22 @@ def swiglu(GU: Tensor) -> Tensor:
     out = torch.empty(n, I, dtype=GU.dtype, device=GU.device)
     check(lib.mq_swiglu(GU.data_ptr(), GU.stride(0), n, I, _dt(GU.dtype), out.data_ptr(), I, _stream(GU)), "mq_swiglu")
     return out
+
+
+def swiglu_packed(G: Tensor, U: Tensor) -> PackedTokens:
+    """silu(G) * U (both (n, I) bf16/fp16, rows may be strided: e.g. the two halves of one stacked GEMM output), same
+    roundings as `swiglu`, written straight into the packed-token layout `hessian_syrk_packed_` reads."""
+    _dev(G, U)
+    lib = _lib.load()
+    if (G.dim() != 2 or G.shape != U.shape or G.dtype != U.dtype or G.dtype not in (torch.bfloat16, torch.float16)
+            or G.shape[1] % 8 or G.stride(1) != 1 or U.stride(1) != 1):
+        raise ValueError("G and U must be (n, I) bf16/fp16 of one dtype with unit column stride and I % 8 == 0")
+    n, I = G.shape
+    nbytes = lib.mq_packed_tokens_bytes(n, I)
+    out = torch.empty(max(nbytes, 16) // 2, dtype=G.dtype, device=G.device)
+    check(lib.mq_swiglu_packed(G.data_ptr(), G.stride(0) if n > 1 else I, U.data_ptr(), U.stride(0) if n > 1 else I, n, I,
+                               _dt(G.dtype), out.data_ptr(), _stream(G)), "mq_swiglu_packed")
+    return PackedTokens(out, n, I, G.dtype)
 
 
 def gemm_f32_(A, sam, sak, B, sbk, sbn, Cm, M, N, K, alpha=1.0, beta=0.0, tri=0, ktrim=0):

@@ -40,7 +40,7 @@ def first_differences_tie_distance(q, ref):
     return ref["tie_distance"][rows, first[rows]]
 
 
-def _run_case(case, dev, chunks=3, code_gate=0.999, same_h_gate=0.9995, tie_tol=1e-3):
+def _run_case(case, dev, chunks=3, code_gate=0.999, same_h_gate=0.999, tie_tol=1e-3, max_rows_differing=0.03):
     _say(f"case {case.name} W{tuple(case.W.shape)} X{tuple(case.X.shape)} g={case.group_size} act={case.act_order}")
     h = GPTQ(_layer(case.W, dev), group_size=case.group_size, sym=True, rel_damp=case.rel_damp,
              block_size=case.block_size, quantization_order="activation" if case.act_order else "default")
@@ -58,8 +58,11 @@ def _run_case(case, dev, chunks=3, code_gate=0.999, same_h_gate=0.9995, tie_tol=
                             block_size=case.block_size, act_order=case.act_order)
     match = (q.cpu() == ref["qweight"]).float().mean().item()
     # The same comparison with the Hessian taken out of the equation: the oracle run on the very matrix the GPU
-    # accumulated.  What is left is factorisation + loop, gated tighter than the end-to-end figure; and every row's
-    # first difference must sit on a rounding decision the oracle itself found close.
+    # accumulated.  What is left is factorisation + loop.  The fraction of equal codes is a blunt figure here -- one
+    # flipped decision early in a row changes most of that row, 0.02-0.05% of a 2048-row matrix (measured on the full
+    # config-1 problem: 15-18 such rows, 99.93-99.96% equal codes) -- so the gate on it stays at 99.9% and the sharp
+    # checks are structural: few rows differ at all, and every row's first difference sits on a rounding decision the
+    # oracle itself found to be a tie (|x/s + zero + 0.5 - integer| of a few 1e-6; a defect flips decisions that are not).
     # (act-order: diag(H) holds exactly equal fp32 values once there are a thousand channels, and torch.argsort leaves
     # their order open -- the CPU's and the device's sort may differ there.  The oracle gets the order the device chose,
     # after checking that it is a valid descending order of that diagonal.)
@@ -76,6 +79,7 @@ def _run_case(case, dev, chunks=3, code_gate=0.999, same_h_gate=0.9995, tie_tol=
     _say(f"  same Hessian: code match {match_same:.6f}; rows that differ {td.numel()}, largest tie distance at a first "
          f"difference {td.max().item() if td.numel() else 0.0:.2e}")
     assert match_same >= same_h_gate
+    assert td.numel() <= max(1, int(max_rows_differing * q.shape[0]))
     assert td.numel() == 0 or td.max().item() < tie_tol
     Wd = case.W.double()
     e_hip = O.relative_mse(O.dequantize_linear_weight(q.cpu(), s.cpu(), z.cpu()).double(), Wd, H64).item()

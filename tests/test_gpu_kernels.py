@@ -793,7 +793,7 @@ def test_hessian_syrk_tail_round_split(dev):
     from moe_quant_amd import _lib
 
     C, n = 7168, 32768 + 40
-    assert _lib.load().mq_hessian_syrk_workspace_bytes(n, C) > 0 and _lib.load().mq_hessian_syrk_workspace_bytes(8192, C) == 0
+    assert _lib.load().mq_hessian_syrk_workspace_bytes(n, C) > 0
     g = torch.Generator(device=dev).manual_seed(5)
     X = torch.randn(n, C, generator=g, device=dev)
     X[:, synth.outlier_channels(C, 6).to(dev)] *= 20.0
@@ -826,3 +826,94 @@ def test_swiglu_against_the_torch_expression(dev, n, I, dtype):
         ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
         assert ((got.float() - want.float()).abs() <= ulp * want.float().abs() + 1e-30).all()
         assert (got == want).float().mean().item() > 0.99
+
+
+# ---------------------------------------------------------------- packed tokens: gather + re-layout, Hessian, SiLU product
+@pytest.mark.parametrize("n,C", [(1, 8), (37, 264), (300, 512), (1000, 2048)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_pack_tokens_layout_and_gather(dev, n, C, dtype):
+    """Xp[o][c][j] = X[rows[8 o + j]][c], zeros in the padding (tokens to a multiple of 128, channels to a multiple of
+    256); the token-major copy written by the same pass equals X[rows]."""
+    g = torch.Generator(device=dev).manual_seed(n + C)
+    X = torch.randn(3 * n + 5, C, generator=g, device=dev).to(dtype)
+    rows = torch.randint(0, X.shape[0], (n,), generator=g, device=dev)
+    P, Xg = ops.pack_tokens(X, rows, also_token_major=True)
+    assert torch.equal(Xg, X[rows]) and (P.n, P.C, P.dtype) == (n, C, dtype)
+    Cp, npad = (C + 255) // 256 * 256, (n + 127) // 128 * 128
+    full = P.data[: npad * Cp].view(npad // 8, Cp, 8).permute(0, 2, 1).reshape(npad, Cp)
+    want = torch.zeros(npad, Cp, dtype=dtype, device=dev)
+    want[:n, :C] = X[rows]
+    assert torch.equal(full, want)
+    assert torch.equal(ops.unpack_tokens(P), X[rows])
+    P2 = ops.pack_tokens(X)  # no gather
+    assert torch.equal(ops.unpack_tokens(P2), X)
+
+
+@pytest.mark.parametrize("n,C,beta", [(300, 264, 0.0), (4096, 2048, 0.5), (32768 + 40, 7168, 0.25), (1, 512, 0.0),
+                                      (9000, 1536, 1.0)])
+def test_hessian_syrk_packed_vs_fp64(dev, n, C, beta):
+    """The Hessian product on packed tokens against an fp64 product formed on the GPU (1e-5 relative Frobenius, the
+    Hessian gate): few tiles cut into token ranges (C = 2048, 1536, 512), the tail-round split (7168 channels from 32768
+    tokens on), padded channels (264), a single token, accumulation onto an old H."""
+    g = torch.Generator(device=dev).manual_seed(n)
+    X = torch.randn(n, C, generator=g, device=dev)
+    X[:, synth.outlier_channels(C, 7).to(dev)] *= 20.0
+    X = X.to(torch.bfloat16)
+    H0 = torch.randn(C, C, generator=g, device=dev)
+    H0 = H0 + H0.t()
+    H = H0.clone()
+    ops.hessian_syrk_packed_(H, ops.pack_tokens(X), beta, 2.0 / n, mirror=True)
+    ref = torch.zeros(C, C, device=dev, dtype=torch.float64)
+    for s0 in range(0, n, 8192):
+        blk = X[s0:s0 + 8192].double()
+        ref.addmm_(blk.t(), blk)
+    ref = beta * H0.double() + (2.0 / n) * ref
+    err = ((H.double() - ref).norm() / ref.norm()).item()
+    _say(f"packed syrk n={n} C={C}: rel err {err:.2e}")
+    assert err < 1e-5 and torch.equal(H, H.t())
+
+
+def test_hessian_syrk_packed_grouped_and_fp16(dev):
+    """Several Hessians of one width in one call, token counts far apart (a MoE layer's experts), fp16 tokens: each
+    against its own fp64 product, and the handle API (update / update_many on PackedTokens) against plain tensors."""
+    from moe_quant_amd.gptq import GPTQ
+
+    C = 768
+    ns = [256, 5000, 129, 2048 + 3]
+    g = torch.Generator(device=dev).manual_seed(3)
+    Xs = [torch.randn(n, C, generator=g, device=dev).to(torch.float16) for n in ns]
+    Hs = [torch.zeros(C, C, device=dev) for _ in ns]
+    ops.hessian_syrk_packed_grouped_(Hs, [ops.pack_tokens(X) for X in Xs], [0.0] * 4, [2.0 / n for n in ns], mirror=True)
+    for H, X, n in zip(Hs, Xs, ns):
+        ref = (2.0 / n) * (X.double().t() @ X.double())
+        assert ((H.double() - ref).norm() / ref.norm()).item() < 1e-5
+    lin = lambda: torch.nn.Linear(C, 64, bias=False, dtype=torch.float16, device=dev)
+    a, b = [GPTQ(lin(), 128, True) for _ in ns], [GPTQ(lin(), 128, True) for _ in ns]
+    GPTQ.update_many(a, [ops.pack_tokens(X) for X in Xs])
+    GPTQ.update_many(a, [ops.pack_tokens(X[:200]) for X in Xs])
+    a[0].update(ops.pack_tokens(Xs[0][:77]))
+    GPTQ.update_many(b, Xs)
+    GPTQ.update_many(b, [X[:200] for X in Xs])
+    b[0].update(Xs[0][:77])
+    for ha, hb in zip(a, b):
+        assert ha.num_samples == hb.num_samples
+        ha.symmetrize_hessian(), hb.symmetrize_hessian()
+        assert ((ha.H - hb.H).norm() / hb.H.norm()).item() < 2e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,I", [(1, 8), (37, 2048), (700, 520), (0, 64)])
+def test_swiglu_packed_equals_swiglu(dev, n, I, dtype):
+    """The SiLU product written in the packed layout holds the same bits as the token-major kernel's output; gate and
+    up outputs given as the two halves of one stacked matrix (strided rows) or as two matrices."""
+    g = torch.Generator(device=dev).manual_seed(n + I)
+    GU = (torch.randn(n, 2 * I, generator=g, device=dev) * 3).to(dtype)
+    want = ops.swiglu(GU)
+    for G, U in ((GU[:, :I], GU[:, I:]), (GU[:, :I].contiguous(), GU[:, I:].contiguous())):
+        P = ops.swiglu_packed(G, U)
+        assert (P.n, P.C) == (n, I)
+        if n:
+            assert torch.equal(ops.unpack_tokens(P), want)
+            Ip, npad = (I + 255) // 256 * 256, (n + 127) // 128 * 128
+            full = P.data[: npad * Ip].view(npad // 8, Ip, 8).permute(0, 2, 1).reshape(npad, Ip)
+            assert int((full[n:] != 0).sum()) == 0 and int((full[:, I:] != 0).sum()) == 0
