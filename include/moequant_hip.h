@@ -45,7 +45,9 @@ extern "C" {
  *                                   C and ldx even, X 4-byte aligned;
  *          MQ_DT_F32              : upper tiles of the fp32 GEMM core (fp32-accurate products), no workspace.
  *        n == 0 just scales H by beta.
- *   workspace: mq_hessian_syrk_workspace_bytes(n, C) bytes (0 when the tile count alone fills the GPU).
+ *   workspace: mq_hessian_syrk_workspace_bytes(n, C) bytes, 16-byte aligned: partial tiles of token ranges when the
+ *        tile count alone does not fill the GPU, and, for wide Hessians with many 16-bit tokens (n >= 4096, C >= 4096),
+ *        room for the tokens re-laid out for the matrix cores (see mq_pack_tokens below), which the call then does itself.
  * mq_hessian_syrk_bf16 is the same call with x_dtype = MQ_DT_BF16.
  */
 size_t mq_hessian_syrk_workspace_bytes(int n, int C);
@@ -58,9 +60,10 @@ int mq_hessian_syrk_bf16(float* H, long ldh, const void* X, long ldx, int n, int
  * block: the reference loops over forward hooks, one addmm_ per expert, src/gptq.py:97-103 via quant.py:258-277).
  * H, ldh, X, ldx, n, beta, alpha are HOST arrays with one entry per problem; the device pointers they hold follow
  * the rules above; all X share x_dtype.  When every problem has 16-bit tokens, n >= 256 of them and 16-byte aligned
- * rows, up to 16 problems share a launch and no workspace is touched; otherwise each problem runs as a plain
- * mq_hessian_syrk call with the given workspace (mq_hessian_syrk_grouped_workspace_bytes = the largest single
- * requirement).  mq_hessian_syrk_bf16_grouped is the same call with x_dtype = MQ_DT_BF16. */
+ * rows, up to 16 problems share a launch (wide problems with many tokens are re-laid out into the workspace first, one
+ * after another); otherwise each problem runs as a plain mq_hessian_syrk call with the given workspace
+ * (mq_hessian_syrk_grouped_workspace_bytes = the larger of the largest single requirement and the sum of the re-laid
+ * out copies).  mq_hessian_syrk_bf16_grouped is the same call with x_dtype = MQ_DT_BF16. */
 size_t mq_hessian_syrk_grouped_workspace_bytes(int groups, const int* n, int C);
 int mq_hessian_syrk_grouped(int groups, float* const* H, const long* ldh, const void* const* X, int x_dtype,
                             const long* ldx, const int* n, int C, const float* beta, const float* alpha, int mirror,

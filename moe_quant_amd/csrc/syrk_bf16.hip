@@ -1091,9 +1091,20 @@ extern "C" int mq_hessian_syrk_packed_grouped(int groups, float* const* H, const
   const int Cp = pk_pad_channels(C), tiles = Cp / T2, ntri = tiles * (tiles + 1) / 2;
   for (int g0 = 0; g0 < groups; g0 += SYRK_MAX_GROUP) {
     const int cnt = groups - g0 < SYRK_MAX_GROUP ? groups - g0 : SYRK_MAX_GROUP;
+    // Within a launch the problems with the most tokens go first: a workgroup runs the whole token range of its tile, so
+    // with token counts far apart (the experts of a MoE layer) the long tiles should start early and the short ones
+    // fill the launch's last round.
+    int order[SYRK_MAX_GROUP];
+    for (int i = 0; i < cnt; ++i) order[i] = g0 + i;
+    for (int i = 1; i < cnt; ++i)
+      for (int k = i; k > 0 && n[order[k]] > n[order[k - 1]]; --k) {
+        const int tmp = order[k];
+        order[k] = order[k - 1];
+        order[k - 1] = tmp;
+      }
     SyrkPackedTable t;
     for (int i = 0; i < SYRK_MAX_GROUP; ++i) {
-      const int g = g0 + (i < cnt ? i : 0);
+      const int g = order[i < cnt ? i : 0];
       t.H[i] = H[g];
       t.Xp[i] = (const uint16_t*)Xp[g];
       t.ldh[i] = ldh[g];

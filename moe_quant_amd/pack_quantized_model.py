@@ -56,8 +56,12 @@ def pack_weight(weight: dict, bits: int, sym: bool, group_size: Optional[int] = 
     return out
 
 
-def prepare_quantization_config(bits: int, group_size: int, quantize_only_experts: bool) -> Dict[str, Any]:
-    """pack_quantized_model.py:78-109 (takes the three values instead of the argparse namespace)."""
+def prepare_quantization_config(bits, group_size: Optional[int] = None, quantize_only_experts: Optional[bool] = None) -> Dict[str, Any]:
+    """pack_quantized_model.py:78-109.  Called as the reference calls it, with one namespace that carries `bits`,
+    `group_size` and `quantize_only_experts` (the reference's `args`), or with the three values."""
+    if group_size is None and quantize_only_experts is None and hasattr(bits, "bits"):
+        args = bits
+        bits, group_size, quantize_only_experts = args.bits, args.group_size, args.quantize_only_experts
     ignored_modules = ["lm_head"]
     if quantize_only_experts:
         ignored_modules += ["re:.*self_attn.*", "re:.*shared_experts.*", r"re:.*mlp\.(gate|up|gate_up|down)_proj.*"]

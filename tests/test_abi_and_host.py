@@ -66,7 +66,10 @@ def test_pure_size_query_needs_no_gpu():
     from moe_quant_amd import _lib
 
     lib = _lib.load()
-    assert lib.mq_hessian_syrk_workspace_bytes(8192, 7168) == 0  # enough tiles to fill the GPU: no split
+    # wide and long: the tokens are re-laid out into the workspace first (8192 x 7168 16-bit values, no padding needed)
+    assert lib.mq_hessian_syrk_workspace_bytes(8192, 7168) == lib.mq_packed_tokens_bytes(8192, 7168) == 8192 * 7168 * 2
+    assert lib.mq_packed_tokens_bytes(100, 264) == 128 * 512 * 2  # tokens padded to 128, channels to 256
+    assert lib.mq_hessian_syrk_workspace_bytes(2048, 7168) == 0  # enough tiles to fill the GPU, too short to re-lay out
     need = lib.mq_hessian_syrk_workspace_bytes(65536, 2048)  # 36 tiles of 256x256: the token range is split
     assert need > 0 and need % (36 * 256 * 256 * 4) == 0
     assert lib.mq_hessian_syrk_workspace_bytes(0, 128) == 0
@@ -143,3 +146,15 @@ def test_reference_module_names_resolve():
     assert torch.equal(m.quant_utils.dequantize_linear_weight(q, s, z), O.dequantize_linear_weight(q, s, z))
     w = torch.randn(4, 32)
     assert torch.equal(m.quant_utils.get_relative_mse_error(w * 0.9, w), O.relative_mse(w * 0.9, w))
+
+
+def test_prepare_quantization_config_takes_the_reference_namespace():
+    """pack_quantized_model.py:78 passes its argparse namespace; the three values give the same dict."""
+    import argparse
+
+    from moe_quant_amd.pack_quantized_model import prepare_quantization_config
+
+    ns = argparse.Namespace(bits=4, group_size=128, quantize_only_experts=True, other="ignored")
+    a, b = prepare_quantization_config(ns), prepare_quantization_config(4, 128, True)
+    assert a == b and a["config_groups"]["group_0"]["weights"]["group_size"] == 128 and len(a["ignore"]) == 4
+    assert prepare_quantization_config(argparse.Namespace(bits=4, group_size=64, quantize_only_experts=False))["ignore"] == ["lm_head"]
