@@ -379,7 +379,8 @@ template <typename P>
 __device__ __forceinline__ P* shifted(P* p, long bytes) {
   return reinterpret_cast<P*>(reinterpret_cast<uintptr_t>(p) + bytes);
 }
-// smask: which pointers of g point into the input matrix (bit 0: A, 1: B, 2: C, 3: Csrc); the others point into the
+// smask: which pointers of g point into the input matrix (bit 0: A, 1: B, 2: C, 3: Csrc; bit 4, trailing launches:
+// workgroup 0 reads its old tile there too); the others point into the
 // output buffer
 __device__ __forceinline__ void rebase(GemmF32& g, const FactorGroup& grp, int e, int smask) {
   const long dA = grp.dA[e], dS = grp.dS[e];
@@ -548,7 +549,8 @@ __device__ __forceinline__ void trail_diag_body(GemmF32 g, int total, GemmF32 gi
     // (the last tile of the trailing update's upper-triangle order: the other workgroups cover total-1 tiles)
     // the whole tile goes to the S position: what lies left of a row's diagonal lands in that row's Xt or unused
     // columns, and the Xt part is cleared next
-    diag_tile_update(buf, A, ld, i1, g.Csrc ? g.Csrc : A, g.Csrc ? g.ldcs : ld);
+    const bool from_s = g.Csrc && (smask & 16);  // nothing has written this tile yet
+    diag_tile_update(buf, A, ld, i1, from_s ? g.Csrc : A, from_s ? g.ldcs : ld);
     __syncthreads();
     // Xt starts at zero in its 32x32 tiles below the diagonal ones (those are written whole by the elimination)
     for (int idx2 = threadIdx.x; idx2 < (NB - SB) * (NB / 4); idx2 += 256) {
@@ -766,24 +768,27 @@ struct FactorPlan {
 
   // The trailing launch of step s: fills T, returns its number of workgroups.
   // The trailing update A[0:i1,0:i1] -= P P^T with one 128-wide panel is bound by reading and writing the
-  // trailing matrix, so after the first step (which also carries the matrix from S to A) the panels go in
-  // trail_panels() at a time.  Only block column b-1 has to be complete for the next panel, and workgroup 0
-  // owns its diagonal tile.  Steps in between (column_only): the j panels block column b-1 still lacks --
-  // this one and the j-1 before it, neighbours in memory, A[:, i1 : i1+128j], one product with K = 128j --
-  // into that block column alone, and already into the diagonal tile after the next one, (b-2, b-2).  Every
-  // trail_panels()-th step: the last trail_panels() panels into every tile but (b-1, b-1), which had all but
+  // trailing matrix, so the panels go in trail_panels() at a time.  Only block column b-1 has to be complete for the
+  // next panel, and workgroup 0 owns its diagonal tile.  Steps in between (column_only): the j panels block column
+  // b-1 still lacks -- this one and the j-1 before it, neighbours in memory, A[:, i1 : i1+128j], one product with
+  // K = 128j -- into that block column alone, and already into the diagonal tile after the next one, (b-2, b-2).
+  // Every trail_panels()-th step: the last trail_panels() panels into every tile but (b-1, b-1), which had all but
   // this panel one step early and takes this one from workgroup 0 as always.
+  // Out of place, no launch exists only to carry the matrix from S to A: through the first trail_panels() steps a tile
+  // is written for the first time by whichever launch updates it, and that launch takes the old values from S -- the
+  // block column and the early diagonal tile of a column-only step, every tile of the first full update; workgroup 0
+  // reads S at step 0 alone (from step 1 on its tile is the one the step before wrote early).
   // (2, 3, 4, 6 panels: 306, 311, 314, 315 linears/s at four streams against 286 with one; a single
   // factorisation takes 3.21 -> 3.28 ms with four, the steps in between leave the chip idle.)
   int trail(int s, TrailLaunch& T) const {
     const int b = B - 1 - s, i1 = b * NB, G = grp.n;
     float* P = A + i1;
-    const bool first = (b == B - 1) && !in_place;
     const int TP = trail_panels();
-    const int j = s >= 1 ? (s - 1) % TP + 1 : 1;  // panels owed to block column b-1 (step 0: the plain update)
-    const int column_only = s >= 1 && j < TP;
+    const int j = s % TP + 1;  // panels owed to block column b-1
+    const int column_only = j < TP;
+    const bool fresh = !in_place && s < TP;  // the tiles of this launch (workgroup 0's aside) hold nothing yet
     GemmF32 trail{P, P, A, ld, 1, 1, ld, ld, i1, i1, j * NB, -1.f, 1.f, 1, 0, 1, 0, 0, 0};
-    if (first) {
+    if (fresh) {
       trail.Csrc = S0;
       trail.ldcs = lds;
     }
@@ -792,7 +797,8 @@ struct FactorPlan {
     int t1 = 0;
     GemmF32 g1 = trail;
     if (!chol && b <= B - 2) g1 = inv_first(b, t1);  // rows > b of the inverse are complete
-    T = TrailLaunch{trail, total, g1, t1, kc_of(C - i1 - NB), A, ld, i1, column_only, others, first ? 8 : 0, Rd};
+    T = TrailLaunch{trail, total, g1, t1, kc_of(C - i1 - NB), A, ld, i1, column_only, others,
+                    (fresh ? 8 : 0) | (fresh && s == 0 ? 16 : 0), Rd};
     return G * (1 + t1 + others);
   }
 
