@@ -57,6 +57,31 @@ def parse():
     return ap.parse_args()
 
 
+def kernel_sources_sha():
+    """Short hash over the library's kernel sources: a profile table records it, so that a table made for other kernels
+    than the ones running shows up in the line that quotes it."""
+    import hashlib
+
+    h = hashlib.sha1()
+    d = os.path.join(ROOT, "moe_quant_amd", "csrc")
+    for f in sorted(os.listdir(d)):
+        if f.endswith((".hip", ".hpp")):
+            h.update(f.encode())
+            h.update(open(os.path.join(d, f), "rb").read())
+    return h.hexdigest()[:12]
+
+
+def profile_sources_sha(file="config1_bench_hbm_traffic"):
+    """The kernel-source hash recorded in profiles/<file>.md (a line `kernel sources: <hash>`), or None."""
+    path = os.path.join(ROOT, "profiles", file + ".md")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("kernel sources:"):
+            return line.split(":", 1)[1].strip()
+    return None
+
+
 def traffic_from_profiles(call, file="config1_bench_hbm_traffic", **keys):
     """HBM bytes per call of `call` for the configuration `keys`, from the table of measured traffic committed in
     profiles/<file>.md (lines of the form `| call | C=7168 G=8 panels=8 | 2.4e10 | ...`, made by rocprofv3 --pmc runs of
@@ -914,6 +939,7 @@ def main():
         "traffic": traffic,
         "traffic_source": "profiles/config1_bench_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
                           "command, looked up by C, group and panel batch; not re-measured by this run)",
+        "traffic_table_made_for_these_kernel_sources": profile_sources_sha() == kernel_sources_sha(),
         "algorithmic_flop_per_launch": flop_factor * Gq,
         "ms_per_launch": round(t_factor_g * Gq, 4),
     }
