@@ -26,12 +26,13 @@ PEAK_HBM = 8000.0  # GB/s
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--steps", type=int, default=96)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--streams", type=int, default=3,
                     help="groups of independent linears are queued round-robin on this many HIP streams")
-    ap.add_argument("--group", type=int, default=8,
+    ap.add_argument("--group", type=int, default=16,
                     help="independent linears per grouped library call (1 = one linear per call, as a lone GPTQ handle runs)")
+    ap.add_argument("--moe-group", type=int, default=8, help="experts per grouped call in the MoE-layer workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink config 1 (debug only; 1.0 is the benchmark)")
     ap.add_argument("--workload", default="config1", choices=["config1", "config2", "config4", "config5", "moe_layer", "gemm", "syrk", "overlap"],
@@ -336,7 +337,8 @@ def moe_layer_run(args, with_cpu_oracle=True):
     quantize_moe_layer(x[:4096], ids[:4096] % 2, experts[:2])
     counts = torch.bincount(ids.flatten(), minlength=args.experts)
     check = torch.argsort(counts, descending=True)[: args.check_experts].tolist() if args.check_experts else []
-    res = quantize_moe_layer(x, ids, experts, keep_codes=check, overlap=not getattr(args, "no_overlap", False))
+    res = quantize_moe_layer(x, ids, experts, keep_codes=check, overlap=not getattr(args, "no_overlap", False),
+                             group=getattr(args, "moe_group", 8))
     C, I = x.shape[1], experts[0].gate.shape[0]
     n_e = torch.tensor(res.tokens_per_expert, dtype=torch.float64)
     flop_syrk = float((n_e * (C * (C + 1) + I * (I + 1))).sum())
