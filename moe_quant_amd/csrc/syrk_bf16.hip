@@ -425,31 +425,49 @@ __device__ __forceinline__ void syrk_dma_tile(float* __restrict__ H, long ldh, c
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
-          acc[i][j] = mfma16<F16>(__builtin_bit_cast(bf16x8n, va[i]), __builtin_bit_cast(bf16x8n, vb[j]), acc[i][j]);
+          acc[i][j] = mfma16<F16>(__builtin_bit_cast(bf16x8n, vb[j]), __builtin_bit_cast(bf16x8n, va[i]), acc[i][j]);
     }
   }
 #undef MQ_SYRK_ISSUE
 
+  // The products were issued with the operands swapped (block rows = channels of the column tile), so of every 32x32
+  // block a lane holds four runs of four consecutive COLUMNS of one row of H: 16-byte accesses where H allows them.
   const int lr = lane & 31, lk = lane >> 5;
   float* out = partial ? ws + ((long)split * pl.ntail + (L - pl.head)) * (T2 * T2) : H;
+  const bool vec = partial || ((((uintptr_t)H) & 15) == 0 && (ldh & 3) == 0 && (C & 3) == 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 4; ++i) {
+    const int r = wm * 128 + i * 32 + lr;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int c = co + j * 32 + lr;
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+      for (int g = 0; g < 4; ++g) {
+        const int c = co + j * 32 + 8 * g + 4 * lk;
+        const floatx16& a = acc[i][j];
         if (partial) {
-          out[r * T2 + c] = acc[i][j][v];
+          *reinterpret_cast<float4*>(out + r * T2 + c) = float4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
         } else if (m0 + r < C && n0 + c < C) {
           float* q = H + (long)(m0 + r) * ldh + n0 + c;
-          float val = alpha * acc[i][j][v];
-          if (beta != 0.f) val = fmaf(beta, *q, val);
-          *q = val;
+          if (vec) {
+            float4 val = {alpha * a[4 * g], alpha * a[4 * g + 1], alpha * a[4 * g + 2], alpha * a[4 * g + 3]};
+            if (beta != 0.f) {
+              const float4 o = *reinterpret_cast<const float4*>(q);
+              val.x = fmaf(beta, o.x, val.x), val.y = fmaf(beta, o.y, val.y), val.z = fmaf(beta, o.z, val.z),
+              val.w = fmaf(beta, o.w, val.w);
+            }
+            *reinterpret_cast<float4*>(q) = val;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n0 + c + e < C) {
+                float val = alpha * a[4 * g + e];
+                if (beta != 0.f) val = fmaf(beta, q[e], val);
+                q[e] = val;
+              }
+          }
         }
       }
-    }
+  }
 }
 
 template <bool F16>
@@ -633,7 +651,7 @@ __device__ __forceinline__ void syrk_packed_tile(float* __restrict__ H, long ldh
       const unsigned char* nxt = smem + ((kt + 1) % PK_NST) * PK_STAGE;
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        acc[m >> 1][m & 1] = mfma16<F16>(fa0[m >> 1], fb0[m & 1], acc[m >> 1][m & 1]);
+        acc[m >> 1][m & 1] = mfma16<F16>(fb0[m & 1], fa0[m >> 1], acc[m >> 1][m & 1]);
         if (m < 4) fa1[m] = *reinterpret_cast<const bf16x8n*>(stg + 2 * PK_PLANE + a_off + m * 512);
         else if (m < 6) fb1[m - 4] = *reinterpret_cast<const bf16x8n*>(stg + 2 * PK_PLANE + b_off + (m - 4) * 512);
         else issue(kt + PK_NST - 1, 2 + (m - 6));
@@ -645,7 +663,7 @@ __device__ __forceinline__ void syrk_packed_tile(float* __restrict__ H, long ldh
       asm volatile("" ::: "memory");
 #pragma unroll
       for (int m = 0; m < 8; ++m) {
-        acc[m >> 1][m & 1] = mfma16<F16>(fa1[m >> 1], fb1[m & 1], acc[m >> 1][m & 1]);
+        acc[m >> 1][m & 1] = mfma16<F16>(fb1[m & 1], fa1[m >> 1], acc[m >> 1][m & 1]);
         if (m < 4) fa0[m] = *reinterpret_cast<const bf16x8n*>(nxt + a_off + m * 512);
         else if (m < 6) fb0[m - 4] = *reinterpret_cast<const bf16x8n*>(nxt + b_off + (m - 4) * 512);
         else issue(kt + PK_NST, m - 6);
@@ -654,26 +672,45 @@ __device__ __forceinline__ void syrk_packed_tile(float* __restrict__ H, long ldh
     }
     __builtin_amdgcn_s_waitcnt(0x0070);
   }
+  // The products were issued with the operands swapped (block rows = channels of the column tile), so of every 32x32
+  // block a lane holds four runs of four consecutive COLUMNS of one row of H: 16-byte accesses where the rows of H allow
+  // them (the padded channels beyond C are whole runs: C is a multiple of 8 here).
   const int lr = lane & 31, lk = lane >> 5;
   float* out = partial ? ws + ((long)split * pl.ntail + (L - pl.head)) * (T2 * T2) : H;
+  const bool vec = partial || ((((uintptr_t)H) & 15) == 0 && (ldh & 3) == 0 && (C & 3) == 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 4; ++i) {
+    const int r = wm * 128 + i * 32 + lr;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int c = wn * 64 + j * 32 + lr;
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int r = wm * 128 + i * 32 + 8 * (v >> 2) + 4 * lk + (v & 3);
+      for (int g = 0; g < 4; ++g) {
+        const int c = wn * 64 + j * 32 + 8 * g + 4 * lk;
+        const floatx16& a = acc[i][j];
         if (partial) {
-          out[r * T2 + c] = acc[i][j][v];
+          *reinterpret_cast<float4*>(out + r * T2 + c) = float4{a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
         } else if (m0 + r < C && n0 + c < C) {
           float* q = H + (long)(m0 + r) * ldh + n0 + c;
-          float val = alpha * acc[i][j][v];
-          if (beta != 0.f) val = fmaf(beta, *q, val);
-          *q = val;
+          if (vec) {
+            float4 val = {alpha * a[4 * g], alpha * a[4 * g + 1], alpha * a[4 * g + 2], alpha * a[4 * g + 3]};
+            if (beta != 0.f) {
+              const float4 o = *reinterpret_cast<const float4*>(q);
+              val.x = fmaf(beta, o.x, val.x), val.y = fmaf(beta, o.y, val.y), val.z = fmaf(beta, o.z, val.z),
+              val.w = fmaf(beta, o.w, val.w);
+            }
+            *reinterpret_cast<float4*>(q) = val;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n0 + c + e < C) {
+                float val = alpha * a[4 * g + e];
+                if (beta != 0.f) val = fmaf(beta, q[e], val);
+                q[e] = val;
+              }
+          }
         }
       }
-    }
+  }
 }
 template <bool F16>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void syrk_packed_kernel(
