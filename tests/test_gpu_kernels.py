@@ -873,6 +873,32 @@ def test_hessian_syrk_packed_vs_fp64(dev, n, C, beta):
     assert err < 1e-5 and torch.equal(H, H.t())
 
 
+@pytest.mark.parametrize("n,C", [(512, 520), (4100, 4104)])
+def test_hessian_syrk_into_a_view_with_odd_pitch(dev, n, C):
+    """H as a view into a larger buffer: rows 4 bytes off a 16-byte boundary and a pitch that is no multiple of four
+    floats, so the kernels take their element-wise stores; same bits as into a plain matrix, nothing written outside."""
+    _say(f"syrk into a strided view n={n} C={C}")
+    g = torch.Generator(device=dev).manual_seed(n + C)
+    X = torch.randn(n, C, generator=g, device=dev).bfloat16()
+    plain = torch.full((C, C), 0.25, device=dev)
+    ops.hessian_syrk_(plain, X, 0.5, 2.0 / n, mirror=True)
+    big = torch.full((C + 2, C + 3), 0.25, device=dev)
+    view = big[1 : C + 1, 2 : C + 2]
+    assert view.data_ptr() % 16 != 0 and view.stride(0) % 4 != 0
+    ops.hessian_syrk_(view, X, 0.5, 2.0 / n, mirror=True)
+    assert torch.equal(view, plain)
+    frame = big.clone()
+    frame[1 : C + 1, 2 : C + 2] = 0.25
+    assert torch.equal(frame, torch.full_like(big, 0.25))
+    P = ops.pack_tokens(X)
+    big.fill_(0.25)
+    ops.hessian_syrk_packed_(view, P, 0.5, 2.0 / n, mirror=True)
+    assert torch.equal(view, plain) or (view - plain).abs().max().item() <= 1e-6 * plain.abs().max().item()
+    frame = big.clone()
+    frame[1 : C + 1, 2 : C + 2] = 0.25
+    assert torch.equal(frame, torch.full_like(big, 0.25))
+
+
 def test_hessian_syrk_packed_grouped_and_fp16(dev):
     """Several Hessians of one width in one call, token counts far apart (a MoE layer's experts), fp16 tokens: each
     against its own fp64 product, and the handle API (update / update_many on PackedTokens) against plain tensors."""
